@@ -86,6 +86,12 @@ class ModelConfig:
     linear_value_head_dim: int = 0
     linear_conv_kernel_dim: int = 4
 
+    # -- per-layer stacks (vurizen): every layer carries its own mixer and
+    # feed-forward description; the flat fields above hold the first layer's
+    # values only so that sizing helpers have something to read ----------------
+    layer_specs: Optional[List[Dict[str, Any]]] = None
+    residual_mult: float = 1.0
+
     raw: Dict[str, Any] = field(default_factory=dict, repr=False)
 
     @property
@@ -99,6 +105,42 @@ class ModelConfig:
     @property
     def is_mla(self) -> bool:
         return self.kv_lora_rank > 0
+
+    # -- cache geometry per local layer (the engine sizes its pools from these) --
+
+    def latent_cache_dims(self, start: int, end: int) -> List[tuple]:
+        """(latent rank, rotated-key width) of every layer in [start, end) that
+        OWNS a compressed-latent cache entry. Layers that read another layer's
+        entry (vurizen `kv_from`) and non-latent layers are left out."""
+        if self.layer_specs is not None:
+            return [
+                (int(sp["mixer"]["kv_rank"]), int(sp["mixer"]["rot_dim"]))
+                for sp in self.layer_specs[start:end]
+                if sp["type"] == "latent_attention"
+                and sp["mixer"].get("kv_from") is None
+            ]
+        if not self.is_mla:
+            return []
+        return [(self.kv_lora_rank, self.qk_rope_head_dim)] * (end - start)
+
+    def linear_state_shapes(self, start: int, end: int) -> List[tuple]:
+        """(conv-state shape, recurrent-state shape) of every linear-attention
+        layer in [start, end)."""
+        if self.layer_specs is not None:
+            return [
+                ((0,), (int(sp["mixer"]["heads"]), int(sp["mixer"]["dim"]),
+                        int(sp["mixer"]["vdim"])))
+                for sp in self.layer_specs[start:end] if sp["type"] == "gla"
+            ]
+        if not self.has_linear_layers:
+            return []
+        conv_dim = (2 * self.linear_num_key_heads * self.linear_key_head_dim
+                    + self.linear_num_value_heads * self.linear_value_head_dim)
+        n = sum(1 for g in range(start, end)
+                if self.layer_type(g) == "linear_attention")
+        return [((conv_dim, self.linear_conv_kernel_dim - 1),
+                 (self.linear_num_value_heads, self.linear_key_head_dim,
+                  self.linear_value_head_dim))] * n
 
     @property
     def is_dsa(self) -> bool:
@@ -114,6 +156,8 @@ class ModelConfig:
 
     def layer_type(self, layer_idx: int) -> str:
         """'attention' | 'sliding_attention' | 'linear_attention' | 'mla_attention'."""
+        if self.layer_specs is not None:
+            return self.layer_types[layer_idx]
         if self.is_mla:
             return "mla_attention"
         if self.layer_types is not None:
@@ -130,7 +174,69 @@ class ModelConfig:
         return (layer_idx % max(1, self.moe_layer_freq)) == 0
 
     @classmethod
+    def from_layer_list_config(cls, cfg: Dict[str, Any]) -> "ModelConfig":
+        """Configs that describe the stack as a list of layers
+        ({"architecture": ..., "layers": [{"type", "mixer", "mlp"}, ...],
+        "norm": {"eps"}, "residual_mult", "vocab", "width"})."""
+        layers = cfg["layers"]
+        kinds = {"gla": "linear_attention", "latent_attention": "latent_attention"}
+        for sp in layers:
+            if sp["type"] not in kinds:
+                raise ValueError(f"unknown layer type {sp['type']!r}")
+            mlp = sp.get("mlp")
+            if mlp is not None and mlp.get("kind", "moe") != "moe":
+                raise ValueError(f"unknown feed-forward kind {mlp.get('kind')!r}")
+        latent = [sp["mixer"] for sp in layers if sp["type"] == "latent_attention"]
+        linear = [sp["mixer"] for sp in layers if sp["type"] == "gla"]
+        moes = [sp["mlp"] for sp in layers if sp.get("mlp") is not None]
+        first = layers[0]["mixer"]
+        mc = cls(
+            architecture=cfg["architecture"],
+            model_type=str(cfg["architecture"]).lower(),
+            vocab_size=int(cfg["vocab"]),
+            hidden_size=int(cfg["width"]),
+            num_layers=len(layers),
+            num_heads=int(first["heads"]),
+            num_kv_heads=int(first["heads"]),
+            head_dim=int(first["dim"]),
+            rms_norm_eps=float(cfg["norm"]["eps"]),
+            max_position_embeddings=int(cfg.get("max_positions", 1 << 20)),
+            layer_types=[kinds[sp["type"]] for sp in layers],
+            eos_token_ids=[],
+            bos_token_id=None,
+            torch_dtype=cfg.get("torch_dtype", "bfloat16"),
+            layer_specs=layers,
+            residual_mult=float(cfg.get("residual_mult", 1.0)),
+            raw=cfg,
+        )
+        if latent:
+            mc.kv_lora_rank = int(latent[0]["kv_rank"])
+            mc.qk_nope_head_dim = int(latent[0]["dim"])
+            mc.qk_rope_head_dim = int(latent[0]["rot_dim"])
+            mc.v_head_dim = int(latent[0]["vdim"])
+            mc.sliding_window = int(latent[0]["mask"]["size"])
+        if linear:
+            mc.linear_num_key_heads = mc.linear_num_value_heads = int(linear[0]["heads"])
+            mc.linear_key_head_dim = int(linear[0]["dim"])
+            mc.linear_value_head_dim = int(linear[0]["vdim"])
+            mc.linear_conv_kernel_dim = 1
+        if moes:
+            r = moes[0]["router"]
+            mc.num_experts = int(r["experts"])
+            mc.num_experts_per_tok = int(r["top"])
+            mc.moe_intermediate_size = int(moes[0]["expert"]["ff"])
+            mc.intermediate_size = mc.moe_intermediate_size
+            mc.scoring_func = "sigmoid"
+            mc.routed_scaling_factor = float(r.get("scale", 1.0))
+            g = r.get("groups") or {}
+            mc.n_group = int(g.get("count", 0))
+            mc.topk_group = int(g.get("keep", 0))
+        return mc
+
+    @classmethod
     def from_hf_config(cls, cfg: Dict[str, Any]) -> "ModelConfig":
+        if "architecture" in cfg and isinstance(cfg.get("layers"), list):
+            return cls.from_layer_list_config(cfg)
         arch = (cfg.get("architectures") or ["LlamaForCausalLM"])[0]
         num_heads = cfg.get("num_attention_heads", 32)
         hidden = cfg.get("hidden_size", 4096)

@@ -34,6 +34,33 @@ class ForwardMeta:
     # host-side max of seq_lens (avoids a device sync when picking the
     # flash-decoding partition count)
     max_seq_len: int = 0
+    # derived per-token tables for packed-sequence kernels (built on first
+    # use, shared by every layer of the forward)
+    _token_seq: Optional[torch.Tensor] = None
+    _query_bounds: Optional[torch.Tensor] = None
+
+    def token_seq(self) -> Optional[torch.Tensor]:
+        """[T] int32: the batch row each packed token belongs to. None for a
+        decode batch (token i is row i)."""
+        if not self.is_prefill:
+            return None
+        if self._token_seq is None:
+            B = self.query_lens.shape[0]
+            self._token_seq = torch.repeat_interleave(
+                torch.arange(B, dtype=torch.int32, device=self.query_lens.device),
+                self.query_lens.long(), output_size=self.num_tokens,
+            )
+        return self._token_seq
+
+    def query_bounds(self) -> Optional[torch.Tensor]:
+        """[B+1] int32 prefix sums of query_lens (None for a decode batch)."""
+        if not self.is_prefill:
+            return None
+        if self._query_bounds is None:
+            self._query_bounds = torch.nn.functional.pad(
+                torch.cumsum(self.query_lens, 0), (1, 0)
+            ).to(torch.int32)
+        return self._query_bounds
 
     @property
     def num_tokens(self) -> int:

@@ -1,0 +1,87 @@
+"""Sliding-window attention over a compressed latent cache.
+
+Per token the cache holds one row [latent c (RMS-normed) | rotated key part]
+shared by all heads; a head's key is [W_uk c | rotated part] and its value
+W_uv c. Attention runs absorbed, as the DeepSeek MLA path of this package
+does: queries are folded through W_uk into the latent space (fp32), scores and
+softmax are fp32 over the cache rows, and the weighted latent sum is expanded
+through W_uv afterwards. Differences from models/deepseek_v3.MLAAttention,
+all parameters: a sliding window (a token sees itself and window - 1 tokens
+before it), separate W_uk / W_uv, rotate-half pairing on the first rot_dims
+dimensions of the rotated part with a YaRN frequency ramp whose softmax scale
+is left untouched, and a layer may read ANOTHER layer's cache rows
+(`cache_layer_idx` of the owner) with its own queries and up-projections.
+"""
+
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+import torch.nn as nn
+
+from .. import ops
+from ..parallel.layers import MergedColumnParallelLinear, RowParallelLinear
+from .forward_meta import ForwardMeta
+from .rope import yarn_ramp_frequencies
+
+
+class LatentWindowAttention(nn.Module):
+    def __init__(self, hidden_size: int, heads: int, nope_dim: int, rot_width: int,
+                 value_dim: int, rank: int, window: int, scale: float,
+                 norm_eps: float, cache_layer_idx: int, owns_cache: bool,
+                 rot_dims: Optional[int] = None, rot_base: float = 10000.0,
+                 rot_scaling: Optional[dict] = None):
+        super().__init__()
+        self.heads, self.dn, self.dr, self.dv = heads, nope_dim, rot_width, value_dim
+        self.rank, self.window, self.scale = rank, int(window), float(scale)
+        self.eps = norm_eps
+        self.cache_layer_idx = cache_layer_idx
+        self.owns_cache = owns_cache
+        self.rot_dims = rot_dims if rot_dims is not None else rot_width
+        sc = rot_scaling or {}
+        self._freq, self._mult = yarn_ramp_frequencies(
+            self.rot_dims, rot_base, float(sc.get("factor", 1.0)),
+            float(sc.get("original", 0.0)), float(sc.get("fast", 32.0)),
+            float(sc.get("slow", 1.0)),
+        )
+        sizes = [heads * (nope_dim + rot_width)]
+        if owns_cache:
+            sizes.append(rank + rot_width)
+            self.latent_norm = nn.Parameter(torch.empty(rank), requires_grad=False)
+        # queries (and, for a layer with a cache of its own, the down
+        # projection to latent + rotated key part) in one GEMM
+        self.in_proj = MergedColumnParallelLinear(hidden_size, sizes)
+        self.w_uk = nn.Parameter(torch.empty(heads, nope_dim, rank), requires_grad=False)
+        self.w_uv = nn.Parameter(torch.empty(heads, value_dim, rank), requires_grad=False)
+        self.o_proj = RowParallelLinear(heads * value_dim, hidden_size)
+        self._f32 = None  # (freq, w_uk fp32, w_uv fp32) on the run device
+
+    def _constants(self, device):
+        if self._f32 is None or self._f32[0].device != device:
+            self._f32 = (self._freq.to(device), self.w_uk.float().contiguous(),
+                         self.w_uv.float().contiguous())
+        return self._f32
+
+    def invalidate_constants(self) -> None:
+        self._f32 = None
+
+    def forward(self, x: torch.Tensor, meta: ForwardMeta) -> torch.Tensor:
+        T, H = x.shape[0], self.heads
+        freq, w_uk, w_uv = self._constants(x.device)
+        parts = self.in_proj.split_output(self.in_proj(x))
+        q = parts[0].view(T, H, self.dn + self.dr)
+        cache = meta.mla_cache.layer(self.cache_layer_idx)
+        if self.owns_cache:
+            ops.latent_kv_store(parts[1], self.latent_norm, self.eps, freq,
+                                self._mult, self.rot_dims, meta.positions,
+                                meta.slot_mapping, cache, self.rank)
+        q_rot = ops.rope_rows(q, self.dn, self.dr, freq, self._mult,
+                              self.rot_dims, meta.positions)
+        q_lat = torch.einsum("thd,hdr->thr", q[..., : self.dn].float(), w_uk)
+        out_lat = ops.latent_window_attention(
+            q_lat.contiguous(), q_rot, cache, meta.block_tables,
+            meta.token_seq(), meta.positions, self.window, self.scale,
+        )
+        attn = torch.einsum("thr,hvr->thv", out_lat, w_uv).to(x.dtype)
+        return self.o_proj(attn.reshape(T, H * self.dv))

@@ -42,6 +42,25 @@ class RMSNorm(nn.Module):
         return ops.fused_add_rmsnorm(x, residual, self.weight, self.eps)
 
 
+class ResidualLayerNorm(nn.Module):
+    """Layer norm (weight and bias) over an fp32 residual stream, fused with
+    the scaled update that precedes it: resid += mult * scale * y, then
+    (resid - mean) / sqrt(var + eps) * weight + bias in the activation dtype.
+    For pre-norm stacks that keep the residual in fp32 and scale each branch
+    (layer scale, residual multiplier)."""
+
+    def __init__(self, hidden_size: int, eps: float):
+        super().__init__()
+        self.weight = nn.Parameter(torch.empty(hidden_size), requires_grad=False)
+        self.bias = nn.Parameter(torch.empty(hidden_size), requires_grad=False)
+        self.eps = eps
+
+    def forward(self, resid: torch.Tensor, y: Optional[torch.Tensor] = None,
+                scale: Optional[torch.Tensor] = None, mult: float = 1.0):
+        return ops.add_layernorm(resid, y, scale, mult, self.weight, self.bias,
+                                 self.eps, self.weight.dtype)
+
+
 class LlamaAttention(nn.Module):
     def __init__(self, cfg: ModelConfig, layer_idx: int, local_layer_idx: int):
         super().__init__()

@@ -62,7 +62,7 @@ class MoERouter(nn.Module):
             topk_ids = select.topk(self.top_k, dim=-1).indices
             topk_w = scores.gather(1, topk_ids)
             if self.norm_topk_prob:
-                topk_w = topk_w / topk_w.sum(dim=-1, keepdim=True).clamp_min(1e-20)
+                topk_w = topk_w / (topk_w.sum(dim=-1, keepdim=True) + 1e-20)
             topk_w = topk_w * self.routed_scaling_factor
         else:
             probs = logits.softmax(dim=-1)
@@ -115,6 +115,9 @@ class FusedMoE(nn.Module):
         # per-expert token counters, graph-safe (fixed-shape scatter_add
         # on a buffer that exists before capture). None = disabled, free.
         self.routing_counts: Optional[torch.Tensor] = None
+        # stacks that add the expert sum into an fp32 residual take the
+        # kernel's fp32 accumulator as it is
+        self.fp32_output = False
 
     def enable_routing_stats(self) -> None:
         self.routing_counts = torch.zeros(
@@ -209,7 +212,10 @@ class FusedMoE(nn.Module):
                 valid, local, torch.full_like(local, self.num_local_experts)
             )
             topk_w = topk_w * valid
-        if x.is_cuda:
+        # the grouped-GEMM kernels take bf16 activations and tile H by 32 and
+        # I by 64; other types and sizes run the per-expert loop below
+        if x.is_cuda and x.dtype == torch.bfloat16 and H % 32 == 0 \
+                and self.intermediate_size % 64 == 0:
             if self.fp8:
                 out = ops.fused_moe_forward_fp8(
                     x, self.w_gate_up_fp8, self.w_gu_scale,
@@ -223,7 +229,7 @@ class FusedMoE(nn.Module):
                 )
             if self.ep_size > 1:
                 out = self._comm.tp_all_reduce(out)
-            return out.to(x.dtype)
+            return out if self.fp32_output else out.to(x.dtype)
         out = torch.zeros(T, H, dtype=torch.float32, device=x.device)
         flat_ids = topk_ids.reshape(-1)              # [T*k]
         flat_w = topk_w.reshape(-1)
@@ -243,13 +249,16 @@ class FusedMoE(nn.Module):
                 gate = h[:, :I].clamp(max=self.act_limit)
                 up = h[:, I:].clamp(min=-self.act_limit, max=self.act_limit)
                 h = (up + 1.0) * (gate * torch.sigmoid(gate * 1.702))
+            elif h.is_cuda and h.dtype != torch.bfloat16:
+                I = self.intermediate_size
+                h = F.silu(h[:, :I]) * h[:, I:]
             else:
                 h = ops.silu_and_mul(h)
             ye = F.linear(h, self._expert_down(e, h.dtype)).float()  # [n_e, H]
             out.index_add_(0, toks, ye * flat_w[sel].unsqueeze(-1))
         if self.ep_size > 1:
             out = self._comm.tp_all_reduce(out)
-        return out.to(x.dtype)
+        return out if self.fp32_output else out.to(x.dtype)
 
 
 class MoEBlock(nn.Module):

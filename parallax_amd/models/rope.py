@@ -92,6 +92,40 @@ def compute_inv_freq_and_scale(
     return inv_freq, 1.0
 
 
+def yarn_ramp_frequencies(
+    dims: int,
+    base: float,
+    factor: float = 1.0,
+    original: float = 0.0,
+    fast: float = 32.0,
+    slow: float = 1.0,
+    ramp_top: Optional[int] = None,
+) -> Tuple[torch.Tensor, float]:
+    """Per-pair rotation frequencies with a YaRN ramp, for kernels that turn
+    positions into angles themselves: f_i = base^(-2i/dims), i < dims/2,
+    blended as f_i/factor * ramp_i + f_i * (1 - ramp_i) where ramp rises
+    linearly from pair lo to pair hi,
+        lo = max(floor(d(fast)), 0),  hi = min(ceil(d(slow)), ramp_top),
+        d(t) = dims * ln(original / (2 pi t)) / (2 ln base).
+    ramp_top defaults to dims - 1. Returns (fp32 frequencies computed in
+    float64, the factor 0.1 ln(factor) + 1 that multiplies cos and sin).
+    factor <= 1 or original <= 0 means no scaling."""
+    half = dims // 2
+    idx = torch.arange(half, dtype=torch.float64)
+    f = torch.pow(torch.tensor(float(base), dtype=torch.float64), -2.0 * idx / dims)
+    if not original or factor == 1.0:
+        return f.float(), 1.0
+
+    def d(turns: float) -> float:
+        return dims * math.log(original / (2 * math.pi * turns)) / (2 * math.log(base))
+
+    lo = max(math.floor(d(fast)), 0)
+    hi = min(math.ceil(d(slow)), dims - 1 if ramp_top is None else ramp_top)
+    ramp = torch.clamp((idx - lo) / max(hi - lo, 1e-3), 0.0, 1.0)
+    out = f / factor * ramp + f * (1.0 - ramp)
+    return out.float(), 0.1 * math.log(factor) + 1.0
+
+
 def build_rope_cache_for(cfg: ModelConfig, rot_dim: Optional[int] = None) -> torch.Tensor:
     rot = rot_dim or cfg.head_dim
     inv_freq, mscale = compute_inv_freq_and_scale(

@@ -629,3 +629,15 @@ def sample_tokens(logits, temperatures, top_ps, top_ks, min_ps,
 
 
 apply_penalties = ref.apply_penalties
+
+
+# -- sequence mixers (extension _mix) ------------------------------------------
+from .mix import (  # noqa: E402,F401
+    add_layernorm,
+    gated_rmsnorm,
+    gla_recurrence,
+    has_mix_extension,
+    latent_kv_store,
+    latent_window_attention,
+    rope_rows,
+)

@@ -1,0 +1,249 @@
+// Python bindings of the sequence-mixer kernels (extension parallax_amd.ops._mix):
+// fp32-residual layer norm, sliding-window latent attention, gated linear
+// attention. Every entry point checks shapes and types on the host before a
+// launch; activation tensors are bf16 or float32 (one template instance each).
+
+#include <ATen/hip/HIPContext.h>
+#include <torch/extension.h>
+
+#include <hip/hip_runtime.h>
+
+extern "C" {
+void launch_add_layernorm(float*, const void*, int64_t, int, const void*, float,
+                          const void*, const void*, float, void*, int, int, int,
+                          hipStream_t);
+void launch_latent_kv_store(const void*, int64_t, const void*, float,
+                            const float*, float, int, const int*,
+                            const int64_t*, void*, int, int, int, int,
+                            hipStream_t);
+void launch_rope_rows(float*, const void*, int64_t, int64_t, int, const float*,
+                      float, int, const int*, int, int, int, int, hipStream_t);
+void launch_latent_window_attention(float*, const float*, const float*,
+                                    const void*, const int*, int, const int*,
+                                    const int*, int, int, int, int, int, int,
+                                    float, int, hipStream_t);
+void launch_gla_recurrence(float*, const void*, const void*, const void*,
+                           const void*, int64_t, int64_t, int64_t, int64_t,
+                           const void*, float*, const int64_t*, const int*,
+                           const int*, int, int, int, int, float, float, int,
+                           hipStream_t);
+void launch_gated_rmsnorm(void*, const float*, const void*, int64_t,
+                          const void*, float, int, int, int, int, hipStream_t);
+}
+
+static hipStream_t cur_stream() {
+  return at::hip::getCurrentHIPStream().stream();
+}
+
+static int kind_of(const torch::Tensor& t, const char* what) {
+  TORCH_CHECK(t.is_cuda(), what, " must be on the GPU");
+  if (t.scalar_type() == at::kBFloat16) return 0;
+  if (t.scalar_type() == at::kFloat) return 1;
+  TORCH_CHECK(false, what, " must be bfloat16 or float32");
+  return -1;
+}
+
+#define CHECK_I32(x) \
+  TORCH_CHECK(x.is_cuda() && x.scalar_type() == at::kInt && x.is_contiguous(), #x " must be int32, contiguous, on the GPU")
+#define CHECK_I64(x) \
+  TORCH_CHECK(x.is_cuda() && x.scalar_type() == at::kLong && x.is_contiguous(), #x " must be int64, contiguous, on the GPU")
+#define CHECK_F32C(x) \
+  TORCH_CHECK(x.is_cuda() && x.scalar_type() == at::kFloat && x.is_contiguous(), #x " must be float32, contiguous, on the GPU")
+
+// resid [T, W] fp32 (updated in place when y is given); y [T, W] (row stride
+// free) or empty; scale [W]; weight/bias [W] or empty (no norm); out [T, W].
+void add_layernorm(torch::Tensor resid, torch::Tensor y, torch::Tensor scale,
+                   double mult, torch::Tensor weight, torch::Tensor bias,
+                   double eps, torch::Tensor out) {
+  CHECK_F32C(resid);
+  TORCH_CHECK(resid.dim() == 2);
+  const int rows = resid.size(0), W = resid.size(1);
+  const bool has_y = y.numel() > 0, has_w = weight.numel() > 0;
+  int y_kind = 1, p_kind = 1;
+  int64_t y_stride = 0;
+  if (has_y) {
+    y_kind = kind_of(y, "y");
+    TORCH_CHECK(y.dim() == 2 && y.size(0) == rows && y.size(1) == W &&
+                y.stride(1) == 1);
+    y_stride = y.stride(0);
+    p_kind = kind_of(scale, "scale");
+    TORCH_CHECK(scale.numel() == W && scale.is_contiguous());
+  }
+  if (has_w) {
+    const int wk = kind_of(weight, "weight");
+    TORCH_CHECK(!has_y || wk == p_kind, "scale and weight types differ");
+    p_kind = wk;
+    TORCH_CHECK(weight.numel() == W && bias.numel() == W &&
+                weight.is_contiguous() && bias.is_contiguous() &&
+                bias.scalar_type() == weight.scalar_type());
+    TORCH_CHECK(out.is_cuda() && out.scalar_type() == weight.scalar_type() &&
+                out.is_contiguous() && out.dim() == 2 && out.size(0) == rows &&
+                out.size(1) == W);
+  }
+  launch_add_layernorm(resid.data_ptr<float>(),
+                       has_y ? y.data_ptr() : nullptr, y_stride, y_kind,
+                       has_y ? scale.data_ptr() : nullptr, (float)mult,
+                       has_w ? weight.data_ptr() : nullptr,
+                       has_w ? bias.data_ptr() : nullptr, (float)eps,
+                       has_w ? out.data_ptr() : nullptr, p_kind, rows, W,
+                       cur_stream());
+}
+
+// dkv [T, rank + rot_w]; cache [blocks, block, rank + rot_w]; freq [rot_dims/2]
+void latent_kv_store(torch::Tensor dkv, torch::Tensor norm_w, double eps,
+                     torch::Tensor freq, double mult, int64_t rot_dims,
+                     torch::Tensor positions, torch::Tensor slots,
+                     torch::Tensor cache, int64_t rank) {
+  const int kind = kind_of(dkv, "dkv");
+  TORCH_CHECK(dkv.dim() == 2 && dkv.stride(1) == 1);
+  const int T = dkv.size(0);
+  const int rot_w = dkv.size(1) - rank;
+  TORCH_CHECK(rank > 0 && rot_w >= 0 && rot_dims % 2 == 0 && rot_dims <= rot_w);
+  TORCH_CHECK(cache.is_cuda() && cache.scalar_type() == dkv.scalar_type() &&
+              cache.is_contiguous() && cache.dim() == 3 &&
+              cache.size(2) == rank + rot_w);
+  TORCH_CHECK(norm_w.scalar_type() == dkv.scalar_type() &&
+              norm_w.numel() == rank && norm_w.is_contiguous());
+  CHECK_F32C(freq);
+  TORCH_CHECK(freq.numel() == rot_dims / 2);
+  CHECK_I32(positions);
+  CHECK_I64(slots);
+  TORCH_CHECK(positions.numel() == T && slots.numel() == T);
+  launch_latent_kv_store(dkv.data_ptr(), dkv.stride(0), norm_w.data_ptr(),
+                         (float)eps, freq.data_ptr<float>(), (float)mult,
+                         (int)rot_dims, positions.data_ptr<int>(),
+                         slots.data_ptr<int64_t>(), cache.data_ptr(), (int)rank,
+                         rot_w, T, kind, cur_stream());
+}
+
+// q [T, H, D] (strided view); rotates columns [col0, col0 + rot_w) of every
+// head into out [T, H, rot_w] fp32
+void rope_rows(torch::Tensor out, torch::Tensor q, int64_t col0,
+               torch::Tensor freq, double mult, int64_t rot_dims,
+               torch::Tensor positions) {
+  const int kind = kind_of(q, "q");
+  CHECK_F32C(out);
+  TORCH_CHECK(q.dim() == 3 && out.dim() == 3 && q.stride(2) == 1);
+  const int T = q.size(0), H = q.size(1), rot_w = out.size(2);
+  TORCH_CHECK(out.size(0) == T && out.size(1) == H);
+  TORCH_CHECK(col0 >= 0 && col0 + rot_w <= q.size(2));
+  TORCH_CHECK(rot_dims % 2 == 0 && rot_dims <= rot_w);
+  CHECK_F32C(freq);
+  TORCH_CHECK(freq.numel() == rot_dims / 2);
+  CHECK_I32(positions);
+  TORCH_CHECK(positions.numel() == T);
+  launch_rope_rows(out.data_ptr<float>(), q.data_ptr(), q.stride(0),
+                   q.stride(1), (int)col0, freq.data_ptr<float>(), (float)mult,
+                   (int)rot_dims, positions.data_ptr<int>(), H, rot_w, T, kind,
+                   cur_stream());
+}
+
+// out/q_lat [T, H, rank] fp32, q_rot [T, H, rot_w] fp32, cache [blocks, block,
+// rank + rot_w], block_tables [B, max_blocks] int32, token_seq [T] int32 or
+// empty (token i belongs to sequence i), positions [T] int32
+void latent_window_attention(torch::Tensor out, torch::Tensor q_lat,
+                             torch::Tensor q_rot, torch::Tensor cache,
+                             torch::Tensor block_tables, torch::Tensor token_seq,
+                             torch::Tensor positions, int64_t window,
+                             double scale) {
+  const int kind = kind_of(cache, "cache");
+  CHECK_F32C(out);
+  CHECK_F32C(q_lat);
+  CHECK_F32C(q_rot);
+  TORCH_CHECK(q_lat.dim() == 3 && q_rot.dim() == 3 && cache.dim() == 3 &&
+              cache.is_contiguous());
+  const int T = q_lat.size(0), H = q_lat.size(1), rank = q_lat.size(2);
+  const int rot_w = q_rot.size(2);
+  TORCH_CHECK(q_rot.size(0) == T && q_rot.size(1) == H);
+  TORCH_CHECK(out.sizes() == q_lat.sizes());
+  TORCH_CHECK(cache.size(2) == rank + rot_w, "cache row width");
+  TORCH_CHECK(rank <= 1024, "latent rank above 1024 is not supported");
+  TORCH_CHECK(window >= 1);
+  CHECK_I32(block_tables);
+  CHECK_I32(positions);
+  TORCH_CHECK(block_tables.dim() == 2 && positions.numel() == T);
+  const bool has_seq = token_seq.numel() > 0;
+  if (has_seq) {
+    CHECK_I32(token_seq);
+    TORCH_CHECK(token_seq.numel() == T);
+  } else {
+    TORCH_CHECK(block_tables.size(0) >= T);
+  }
+  launch_latent_window_attention(
+      out.data_ptr<float>(), q_lat.data_ptr<float>(), q_rot.data_ptr<float>(),
+      cache.data_ptr(), block_tables.data_ptr<int>(),
+      (int)block_tables.stride(0), has_seq ? token_seq.data_ptr<int>() : nullptr,
+      positions.data_ptr<int>(), T, H, rank, rot_w, (int)cache.size(1),
+      (int)window, (float)scale, kind, cur_stream());
+}
+
+// q, k, z [T, H*dk] and v [T, H*dv] (row strides free), z_bias [H*dk],
+// state [slots, H, dk, dv] fp32, slots [B] int64, cu [B+1] int32 or empty (one
+// token per sequence), positions [T] int32, o [T, H, dv] fp32
+void gla_recurrence(torch::Tensor o, torch::Tensor q, torch::Tensor k,
+                    torch::Tensor v, torch::Tensor z, torch::Tensor z_bias,
+                    torch::Tensor state, torch::Tensor slots, torch::Tensor cu,
+                    torch::Tensor positions, double inv_tau, double q_scale) {
+  const int kind = kind_of(q, "q");
+  CHECK_F32C(o);
+  CHECK_F32C(state);
+  TORCH_CHECK(state.dim() == 4 && o.dim() == 3);
+  const int H = state.size(1), dk = state.size(2), dv = state.size(3);
+  const int T = o.size(0);
+  TORCH_CHECK(o.size(1) == H && o.size(2) == dv);
+  TORCH_CHECK(dk <= 2048, "gla key dim above 2048 is not supported");
+  for (const torch::Tensor* t : {&q, &k, &z}) {
+    TORCH_CHECK(t->is_cuda() && t->scalar_type() == q.scalar_type() &&
+                t->dim() == 2 && t->size(0) == T && t->size(1) == H * dk &&
+                t->stride(1) == 1);
+  }
+  TORCH_CHECK(v.is_cuda() && v.scalar_type() == q.scalar_type() &&
+              v.dim() == 2 && v.size(0) == T && v.size(1) == H * dv &&
+              v.stride(1) == 1);
+  TORCH_CHECK(z_bias.is_cuda() && z_bias.scalar_type() == q.scalar_type() &&
+              z_bias.numel() == H * dk && z_bias.is_contiguous());
+  CHECK_I64(slots);
+  CHECK_I32(positions);
+  TORCH_CHECK(positions.numel() == T);
+  const int B = slots.numel();
+  const bool has_cu = cu.numel() > 0;
+  if (has_cu) {
+    CHECK_I32(cu);
+    TORCH_CHECK(cu.numel() == B + 1);
+  } else {
+    TORCH_CHECK(B == T, "without cu every sequence brings one token");
+  }
+  launch_gla_recurrence(
+      o.data_ptr<float>(), q.data_ptr(), k.data_ptr(), v.data_ptr(),
+      z.data_ptr(), q.stride(0), k.stride(0), v.stride(0), z.stride(0),
+      z_bias.data_ptr(), state.data_ptr<float>(), slots.data_ptr<int64_t>(),
+      has_cu ? cu.data_ptr<int>() : nullptr, positions.data_ptr<int>(), B, H,
+      dk, dv, (float)inv_tau, (float)q_scale, kind, cur_stream());
+}
+
+// o [T, H, dv] fp32, gate [T, H*dv], weight [dv] -> out [T, H*dv]
+void gated_rmsnorm(torch::Tensor out, torch::Tensor o, torch::Tensor gate,
+                   torch::Tensor weight, double eps) {
+  const int kind = kind_of(gate, "gate");
+  CHECK_F32C(o);
+  TORCH_CHECK(o.dim() == 3);
+  const int T = o.size(0), H = o.size(1), dv = o.size(2);
+  TORCH_CHECK(gate.dim() == 2 && gate.size(0) == T && gate.size(1) == H * dv &&
+              gate.stride(1) == 1);
+  TORCH_CHECK(out.is_cuda() && out.scalar_type() == gate.scalar_type() &&
+              out.is_contiguous() && out.numel() == (int64_t)T * H * dv);
+  TORCH_CHECK(weight.is_cuda() && weight.scalar_type() == gate.scalar_type() &&
+              weight.numel() == dv && weight.is_contiguous());
+  launch_gated_rmsnorm(out.data_ptr(), o.data_ptr<float>(), gate.data_ptr(),
+                       gate.stride(0), weight.data_ptr(), (float)eps, T * H, H,
+                       dv, kind, cur_stream());
+}
+
+PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
+  m.def("add_layernorm", &add_layernorm);
+  m.def("latent_kv_store", &latent_kv_store);
+  m.def("rope_rows", &rope_rows);
+  m.def("latent_window_attention", &latent_window_attention);
+  m.def("gla_recurrence", &gla_recurrence);
+  m.def("gated_rmsnorm", &gated_rmsnorm);
+}

@@ -1,0 +1,139 @@
+"""Sequence-mixer ops: layer norm over an fp32 residual stream, sliding-window
+attention over a compressed latent cache, gated linear attention.
+
+GPU tensors go to the hand-written gfx950 kernels of the in-tree extension
+``parallax_amd.ops._mix`` (bf16 or float32 activations; scores, norms, decays
+and recurrent state always fp32). There is no eager fallback on a GPU: a
+missing extension raises. CPU tensors run the eager torch versions in
+``reference.py`` (CPU engine, tests)."""
+
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from . import reference as ref
+
+_MIX = None
+_MIX_ERR: Optional[str] = None
+
+
+def _mix_ext():
+    global _MIX, _MIX_ERR
+    if _MIX is None and _MIX_ERR is None:
+        try:
+            from . import _mix  # built in-tree (setup.py, PARALLAX_EXT=_mix)
+
+            _MIX = _mix
+        except ImportError as e:
+            _MIX_ERR = str(e)
+    if _MIX is None:
+        raise RuntimeError(
+            "the parallax_amd.ops._mix HIP extension is required on a GPU but "
+            f"is not built (import error: {_MIX_ERR}); build it with "
+            "`PARALLAX_EXT=_mix python setup.py build_ext --inplace`"
+        )
+    return _MIX
+
+
+def has_mix_extension() -> bool:
+    try:
+        _mix_ext()
+        return True
+    except RuntimeError:
+        return False
+
+
+def _empty(like: torch.Tensor, dtype=None) -> torch.Tensor:
+    return like.new_empty(0, dtype=dtype or like.dtype)
+
+
+def add_layernorm(resid, y, scale, mult, weight, bias, eps, out_dtype):
+    """resid [T, W] fp32 <- resid + mult * scale * y (in place; y None = no
+    update), then layer norm with weight and bias -> [T, W] of out_dtype
+    (weight None = no norm, returns None)."""
+    if not resid.is_cuda:
+        return ref.add_layernorm(resid, y, scale, mult, weight, bias, eps, out_dtype)
+    ext = _mix_ext()
+    out = torch.empty(resid.shape, dtype=out_dtype, device=resid.device) \
+        if weight is not None else _empty(resid)
+    ext.add_layernorm(
+        resid, y if y is not None else _empty(resid),
+        scale if y is not None else _empty(resid), float(mult),
+        weight if weight is not None else _empty(resid),
+        bias if weight is not None else _empty(resid), float(eps), out,
+    )
+    return out if weight is not None else None
+
+
+def latent_kv_store(dkv, norm_w, eps, freq, mult, rot_dims, positions,
+                    slot_mapping, cache, rank):
+    """RMS-norm the first `rank` columns of dkv, rotate the rest by position,
+    scatter both as one cache row per token (slot -1 = skip)."""
+    if not dkv.is_cuda:
+        return ref.latent_kv_store(dkv, norm_w, eps, freq, mult, rot_dims,
+                                   positions, slot_mapping, cache, rank)
+    _mix_ext().latent_kv_store(dkv, norm_w, float(eps), freq, float(mult),
+                               int(rot_dims), positions, slot_mapping, cache,
+                               int(rank))
+
+
+def rope_rows(q, col0, rot_w, freq, mult, rot_dims, positions):
+    """q [T, H, D]: columns [col0, col0+rot_w) of every head, rotated on their
+    first rot_dims dimensions, as a new fp32 [T, H, rot_w]."""
+    if not q.is_cuda:
+        return ref.rope_rows(q, col0, rot_w, freq, mult, rot_dims, positions)
+    out = torch.empty(q.shape[0], q.shape[1], rot_w, dtype=torch.float32,
+                      device=q.device)
+    _mix_ext().rope_rows(out, q, int(col0), freq, float(mult), int(rot_dims),
+                         positions)
+    return out
+
+
+def latent_window_attention(q_lat, q_rot, cache, block_tables, token_seq,
+                            positions, window, scale):
+    """Softmax attention of absorbed queries over the paged latent cache with
+    a sliding window: token at position p sees keys p-window+1 .. p of its
+    sequence. q_lat [T, H, rank] fp32, q_rot [T, H, rot_w] fp32, token_seq [T]
+    int32 (None: token i is sequence i). Returns fp32 [T, H, rank]."""
+    if not q_lat.is_cuda:
+        return ref.latent_window_attention(q_lat, q_rot, cache, block_tables,
+                                           token_seq, positions, window, scale)
+    out = torch.empty_like(q_lat)
+    _mix_ext().latent_window_attention(
+        out, q_lat, q_rot, cache, block_tables,
+        token_seq if token_seq is not None
+        else _empty(positions), positions, int(window), float(scale),
+    )
+    return out
+
+
+def gla_recurrence(q, k, v, z, z_bias, state, slots, cu, positions, inv_tau,
+                   q_scale):
+    """Gated-linear-attention recurrence over packed sequences; the fp32
+    state [slots, H, dk, dv] is read (or started from zero at position 0) and
+    written back. cu [B+1] int32 token bounds (None: one token each). Returns
+    fp32 o [T, H, dv]."""
+    if not q.is_cuda:
+        return ref.gla_recurrence(q, k, v, z, z_bias, state, slots, cu,
+                                  positions, inv_tau, q_scale)
+    H, dv = state.shape[1], state.shape[3]
+    o = torch.empty(q.shape[0], H, dv, dtype=torch.float32, device=q.device)
+    _mix_ext().gla_recurrence(
+        o, q, k, v, z, z_bias, state, slots,
+        cu if cu is not None else _empty(positions), positions,
+        float(inv_tau), float(q_scale),
+    )
+    return o
+
+
+def gated_rmsnorm(o, gate, weight, eps, out_dtype):
+    """Per-head RMS norm of o [T, H, dv] (fp32) with a weight shared by heads,
+    times silu(gate) -> [T, H*dv] of out_dtype."""
+    if not o.is_cuda:
+        return ref.gated_rmsnorm(o, gate, weight, eps, out_dtype)
+    T, H, dv = o.shape
+    out = torch.empty(T, H * dv, dtype=out_dtype, device=o.device)
+    _mix_ext().gated_rmsnorm(out, o, gate, weight, float(eps))
+    return out

@@ -556,3 +556,102 @@ def msa_paged_attention_decode(
             p = torch.softmax(logits, dim=-1)
             out[i, h * group:(h + 1) * group] = (p @ vf).to(q.dtype)
     return out
+
+
+# -- sequence mixers: fp32-residual layer norm, latent window attention, GLA ----
+# Eager torch versions of the _mix extension's kernels (CPU engine, oracles of
+# the kernel tests). Same signatures as the wrappers in ops/mix.py.
+
+
+def add_layernorm(resid, y, scale, mult, weight, bias, eps, out_dtype):
+    """resid [T, W] fp32 += mult * scale * y (in place; skipped when y is
+    None); returns layer_norm(resid) * weight + bias in out_dtype (None when
+    weight is None)."""
+    if y is not None:
+        resid.add_(mult * (scale.float() * y.float()))
+    if weight is None:
+        return None
+    mean = resid.mean(-1, keepdim=True)
+    var = ((resid - mean) ** 2).mean(-1, keepdim=True)
+    out = (resid - mean) / torch.sqrt(var + eps) * weight.float() + bias.float()
+    return out.to(out_dtype)
+
+
+def _rotate_rows(x, positions, freq, mult, rot_dims):
+    """x [T, ..., >=rot_dims] fp32; pair (i, i + rot_dims/2)."""
+    half = rot_dims // 2
+    ang = positions.float().unsqueeze(-1) * freq.float()          # [T, half]
+    shape = [x.shape[0]] + [1] * (x.dim() - 2) + [half]
+    c = (torch.cos(ang) * mult).view(shape)
+    s = (torch.sin(ang) * mult).view(shape)
+    u, v = x[..., :half], x[..., half:rot_dims]
+    out = x.clone()
+    out[..., :half] = u * c - v * s
+    out[..., half:rot_dims] = v * c + u * s
+    return out
+
+
+def latent_kv_store(dkv, norm_w, eps, freq, mult, rot_dims, positions,
+                    slot_mapping, cache, rank):
+    x = dkv.float()
+    lat = x[:, :rank]
+    lat = lat / torch.sqrt((lat * lat).mean(-1, keepdim=True) + eps) * norm_w.float()
+    kr = _rotate_rows(x[:, rank:], positions, freq, mult, rot_dims)
+    entry = torch.cat([lat, kr], dim=-1).to(cache.dtype)
+    keep = slot_mapping >= 0
+    flat = cache.view(-1, cache.shape[-1])
+    flat[slot_mapping[keep]] = entry[keep]
+
+
+def rope_rows(q, col0, rot_w, freq, mult, rot_dims, positions):
+    return _rotate_rows(q[..., col0 : col0 + rot_w].float(), positions, freq,
+                        mult, rot_dims).contiguous()
+
+
+def latent_window_attention(q_lat, q_rot, cache, block_tables, token_seq,
+                            positions, window, scale):
+    T, H, rank = q_lat.shape
+    bs = cache.shape[1]
+    out = torch.empty_like(q_lat)
+    pos = positions.tolist()
+    seq = token_seq.tolist() if token_seq is not None else list(range(T))
+    for t in range(T):
+        p = pos[t]
+        lo = max(0, p - window + 1)
+        j = torch.arange(lo, p + 1)
+        bt = block_tables[seq[t]].long()
+        rows = cache[bt[j // bs], j % bs].float()                  # [n, E]
+        s = (q_lat[t] @ rows[:, :rank].T + q_rot[t] @ rows[:, rank:].T) * scale
+        out[t] = torch.softmax(s, dim=-1) @ rows[:, :rank]
+    return out
+
+
+def gla_recurrence(q, k, v, z, z_bias, state, slots, cu, positions, inv_tau,
+                   q_scale):
+    T = q.shape[0]
+    _, H, dk, dv = state.shape
+    qf = q.float().view(T, H, dk) * q_scale
+    kf = k.float().view(T, H, dk)
+    vf = v.float().view(T, H, dv)
+    zf = z.float().view(T, H, dk) + z_bias.float().view(H, dk)
+    alpha = torch.exp(torch.nn.functional.logsigmoid(zf) * inv_tau)
+    o = torch.empty(T, H, dv, dtype=torch.float32)
+    bounds = cu.tolist() if cu is not None else list(range(T + 1))
+    pos = positions.tolist()
+    for b, slot in enumerate(slots.tolist()):
+        t0, t1 = bounds[b], bounds[b + 1]
+        if t0 >= t1:
+            continue
+        S = torch.zeros(H, dk, dv) if pos[t0] == 0 else state[slot].clone()
+        for t in range(t0, t1):
+            S = alpha[t].unsqueeze(-1) * S + kf[t].unsqueeze(-1) * vf[t].unsqueeze(-2)
+            o[t] = torch.einsum("hkv,hk->hv", S, qf[t])
+        state[slot] = S
+    return o
+
+
+def gated_rmsnorm(o, gate, weight, eps, out_dtype):
+    T, H, dv = o.shape
+    x = o / torch.sqrt((o * o).mean(-1, keepdim=True) + eps) * weight.float()
+    g = gate.float().view(T, H, dv)
+    return (x * torch.nn.functional.silu(g)).view(T, H * dv).to(out_dtype)

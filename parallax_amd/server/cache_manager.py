@@ -45,6 +45,10 @@ class CacheManager:
         self.allocator = BlockAllocator(num_blocks, block_size)
         self.radix = BlockRadixCache(self.allocator, block_size, enable=enable_prefix_cache)
         self.slot_allocator = SlotAllocator(num_linear_slots) if num_linear_slots else None
+        # called with the slot id whenever a state slot is handed to a new
+        # request: whoever owns the state tensors clears what the slot's
+        # previous request left there
+        self.on_slot_allocated = None
         self._requests: Dict[str, RequestCacheState] = {}
 
     # -- sizing --------------------------------------------------------------
@@ -104,6 +108,8 @@ class CacheManager:
         )
         if self.slot_allocator is not None:
             state.linear_slot = self.slot_allocator.allocate()
+            if self.on_slot_allocated is not None:
+                self.on_slot_allocated(state.linear_slot)
         self._requests[rid] = state
         return state
 

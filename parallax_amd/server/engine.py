@@ -79,6 +79,9 @@ class EngineArgs:
     enable_routing_stats: bool = False  # per-expert MoE routing counters
     prefill_priority: bool = True       # prefills before decodes in a step
     linear_weight_dtype: str = "auto"   # dense GEMMs: "auto" | "fp8"(W8A8)
+    # recurrent-state slots kept beyond max_batch_size (requests that finish
+    # one step late under async decode still hold theirs)
+    extra_linear_slots: int = 8
 
 
 def partition_layers(num_layers: int, pp_size: int, pp_rank: int) -> Tuple[int, int]:
@@ -124,8 +127,12 @@ class Engine:
             self.model.finalize_weights()
         self.model = self.model.to(device=self.device, dtype=args.dtype)
         # rope cache stays fp32
-        self.model.rope_cache = self.model.rope_cache.float()
+        if getattr(self.model, "rope_cache", None) is not None:
+            self.model.rope_cache = self.model.rope_cache.float()
         self.model.eval()
+        # dtype of the hidden states that enter and leave a shard (designs
+        # that keep their residual stream in fp32 say so on the model class)
+        self.hidden_dtype = getattr(self.model, "hidden_dtype", None) or args.dtype
         if args.moe_weight_dtype == "fp8":
             from ..models.moe import FusedMoE
 
@@ -166,33 +173,32 @@ class Engine:
         if cfg.has_linear_layers:
             from .kv_cache import LinearStateCache
 
-            n_linear = sum(1 for t in self.local_layer_types if t == "linear_attention")
-            conv_dim = (
-                2 * cfg.linear_num_key_heads * cfg.linear_key_head_dim
-                + cfg.linear_num_value_heads * cfg.linear_value_head_dim
-            )
+            shapes = cfg.linear_state_shapes(start, end)
+            if not shapes:  # this shard holds no linear layer: one dummy entry
+                shapes = cfg.linear_state_shapes(0, cfg.num_layers)[:1]
+            n_slots = args.max_batch_size + args.extra_linear_slots
             self.linear_cache = LinearStateCache(
-                max(1, n_linear),
-                conv_state_shape=(conv_dim, cfg.linear_conv_kernel_dim - 1),
-                recurrent_state_shape=(
-                    cfg.linear_num_value_heads, cfg.linear_key_head_dim,
-                    cfg.linear_value_head_dim,
-                ),
+                len(shapes),
+                conv_state_shape=[c for c, _ in shapes],
+                recurrent_state_shape=[r for _, r in shapes],
                 # +1: the last slot is a scratch slot for graph-capture pad
                 # rows (DecodeGraphRunner.linear_scratch_slot); the cache
-                # manager only hands out the first max_batch_size + 8
-                num_slots=args.max_batch_size + 9,
+                # manager only hands out the first n_slots
+                num_slots=n_slots + 1,
                 device=self.device,
                 dtype=args.dtype if args.dtype != torch.float32 else torch.float32,
             )
 
-        self.is_mla = cfg.is_mla
+        self.is_mla = cfg.is_mla or cfg.layer_specs is not None
         if self.is_mla:
-            mla_block_bytes = MLAKVCache.bytes_per_block(
-                end - start, cfg.kv_lora_rank, cfg.qk_rope_head_dim,
+            latent_dims = cfg.latent_cache_dims(start, end)
+            latent_ranks = [r for r, _ in latent_dims]
+            latent_ropes = [d for _, d in latent_dims]
+            mla_block_bytes = max(1, MLAKVCache.bytes_per_block(
+                len(latent_dims), latent_ranks, latent_ropes,
                 args.block_size, args.dtype,
                 index_dim=cfg.index_head_dim if cfg.is_dsa else 0,
-            )
+            ))
             if args.num_kv_blocks:
                 num_blocks = args.num_kv_blocks
             else:
@@ -207,7 +213,7 @@ class Engine:
                 assert self.device.type == "cuda", "fp8 KV needs the HIP kernels"
                 mla_dtype = torch.float8_e4m3fn
             self.kv_cache = MLAKVCache(
-                end - start, cfg.kv_lora_rank, cfg.qk_rope_head_dim,
+                len(latent_dims), latent_ranks, latent_ropes,
                 args.block_size, num_blocks, self.device, mla_dtype,
                 index_dim=cfg.index_head_dim if cfg.is_dsa else 0,
             )
@@ -231,8 +237,13 @@ class Engine:
         self.cache_manager = CacheManager(
             args.block_size, num_blocks,
             enable_prefix_cache=args.enable_prefix_cache and not cfg.has_linear_layers,
-            num_linear_slots=(args.max_batch_size + 8) if cfg.has_linear_layers else 0,
+            num_linear_slots=(args.max_batch_size + args.extra_linear_slots)
+            if cfg.has_linear_layers else 0,
         )
+        if self.linear_cache is not None:
+            # a slot handed to a new request must not carry the state of the
+            # request that held it before
+            self.cache_manager.on_slot_allocated = self.linear_cache.reset_slot
         self.scheduler = Scheduler(
             self.cache_manager,
             max_batch_size=args.max_batch_size,
@@ -248,14 +259,14 @@ class Engine:
             from .graph_runner import DecodeGraphRunner
 
             self.graph_runner = DecodeGraphRunner(
-                self.model, self.kv_cache, self.device, args.dtype,
+                self.model, self.kv_cache, self.device, self.hidden_dtype,
                 max_batch=args.max_batch_size, max_model_len=args.max_model_len,
                 block_size=args.block_size, hidden_size=cfg.hidden_size,
                 is_first_stage=self.comm.is_first_stage,
                 is_last_stage=self.comm.is_last_stage,
                 is_mla=self.is_mla,
                 linear_cache=self.linear_cache,
-                linear_scratch_slot=args.max_batch_size + 8,
+                linear_scratch_slot=args.max_batch_size + args.extra_linear_slots,
             )
         self._pending_adds: List[InitialRequest] = []
         self._inflight = None       # async decode pipelining state
@@ -784,14 +795,14 @@ class Engine:
         positions, input_ids, slot_mapping, block_tables, seq_lens = [], [], [], [], []
         for r in reqs:
             state = self.cache_manager.get(r.rid)
-            pos = r.total_len - 1  # position of the token being fed in
+            tok, pos = r.decode_input()  # the token being fed in, its position
             positions.append(pos)
-            input_ids.append(r.output_token_ids[-1])
+            input_ids.append(tok)
             slot_mapping.extend(
                 slot_mapping_for_positions(state.block_table, pos, 1, self.args.block_size)
             )
             block_tables.append(state.block_table)
-            seq_lens.append(r.total_len)
+            seq_lens.append(pos + 1)
         dev = self.device
         meta = ForwardMeta(
             is_prefill=False,
@@ -821,9 +832,9 @@ class Engine:
         T = meta.num_tokens
         h = self.cfg.hidden_size
         if comm.is_first_stage:
-            hidden = self.model.embed(input_ids).to(self.args.dtype)
+            hidden = self.model.embed(input_ids).to(self.hidden_dtype)
         else:
-            hidden = comm.pp_recv((T, h), self.args.dtype, comm.pp_rank - 1)
+            hidden = comm.pp_recv((T, h), self.hidden_dtype, comm.pp_rank - 1)
         hidden = self.model(hidden, meta)
         if not comm.is_last_stage:
             comm.pp_send(hidden, comm.pp_rank + 1)
@@ -854,7 +865,7 @@ class Engine:
                 for g in groups:
                     T = sum(c.num_tokens for c in g)
                     recvs.append(
-                        comm.pp_irecv((T, h), self.args.dtype, comm.pp_rank - 1)
+                        comm.pp_irecv((T, h), self.hidden_dtype, comm.pp_rank - 1)
                     )
             for i, g in enumerate(groups):
                 hidden_in = None
@@ -873,11 +884,17 @@ class Engine:
 
     def _prefill_group(self, chunks: List[PrefillChunk],
                        hidden_in: Optional[torch.Tensor] = None,
-                       send_slot: Optional[int] = None):
+                       send_slot: Optional[int] = None,
+                       logits_at: Optional[List[int]] = None):
         """Forward one prefill (micro-)batch through the local shard. When
         hidden_in/send_slot are given the PP transport is async (pipelined);
-        otherwise the blocking single-group path runs."""
+        otherwise the blocking single-group path runs. logits_at: packed
+        token indices whose logits are wanted instead of each request's last
+        prompt token (teacher-forced replay)."""
         meta, input_ids = self._build_prefill_meta(chunks)
+        if logits_at is not None:
+            need = torch.tensor(logits_at, dtype=torch.int64, device=self.device)
+            return self._pipeline_forward(meta, input_ids, need)
         keep = torch.tensor(
             [i for i, c in enumerate(chunks) if c.is_last_chunk], dtype=torch.int64
         )
@@ -887,7 +904,7 @@ class Engine:
         if hidden_in is None and send_slot is None:
             return self._pipeline_forward(meta, input_ids, need)
         if comm.is_first_stage:
-            hidden = self.model.embed(input_ids).to(self.args.dtype)
+            hidden = self.model.embed(input_ids).to(self.hidden_dtype)
         else:
             hidden = hidden_in
         hidden = self.model(hidden, meta)
@@ -907,7 +924,7 @@ class Engine:
         if self.graph_runner is None:
             meta, ids = self._build_decode_meta(reqs)
             if self.comm.is_first_stage:
-                hidden = self.model.embed(ids).to(self.args.dtype)
+                hidden = self.model.embed(ids).to(self.hidden_dtype)
             else:
                 hidden = hidden_in
             hidden = self.model(hidden, meta)
@@ -917,15 +934,15 @@ class Engine:
         input_ids, positions, slots, btabs, seq_lens = [], [], [], [], []
         for r in reqs:
             state = self.cache_manager.get(r.rid)
-            pos = r.total_len - 1
+            tok, pos = r.decode_input()
             positions.append(pos)
-            input_ids.append(r.output_token_ids[-1])
+            input_ids.append(tok)
             slots.append(
                 state.block_table[pos // self.args.block_size] * self.args.block_size
                 + pos % self.args.block_size
             )
             btabs.append(state.block_table)
-            seq_lens.append(r.total_len)
+            seq_lens.append(pos + 1)
         lin_slots = None
         if self.linear_cache is not None:
             lin_slots = [
@@ -942,7 +959,7 @@ class Engine:
         hidden_in = None
         if not comm.is_first_stage:
             hidden_in = comm.pp_recv(
-                (len(reqs), self.cfg.hidden_size), self.args.dtype, comm.pp_rank - 1
+                (len(reqs), self.cfg.hidden_size), self.hidden_dtype, comm.pp_rank - 1
             )
         out = self._decode_fwd(reqs, hidden_in)
         if not comm.is_last_stage:
@@ -967,7 +984,7 @@ class Engine:
             if not comm.is_first_stage:
                 for g in groups:
                     recvs.append(
-                        comm.pp_irecv((len(g), h), self.args.dtype, comm.pp_rank - 1)
+                        comm.pp_irecv((len(g), h), self.hidden_dtype, comm.pp_rank - 1)
                     )
             logits_parts = []
             for i, g in enumerate(groups):
@@ -1047,7 +1064,8 @@ class Engine:
         if hasattr(model_cpu, "finalize_weights"):
             model_cpu.finalize_weights()
         self.model = model_cpu.to(device=self.device, dtype=self.args.dtype)
-        self.model.rope_cache = self.model.rope_cache.float()
+        if getattr(self.model, "rope_cache", None) is not None:
+            self.model.rope_cache = self.model.rope_cache.float()
         if self.graph_runner is not None:
             self.graph_runner.model = self.model
             # weights moved: captured graphs reference stale parameter storage
@@ -1067,6 +1085,55 @@ class Engine:
             self.model.finalize_weights()
         self.cache_manager.reset_prefix_cache()
         return n
+
+    # -- teacher-forced replay ------------------------------------------------------------------
+
+    def replay_step(self, entries, end=()) -> Optional[torch.Tensor]:
+        """One engine iteration over GIVEN tokens: nothing is sampled.
+
+        entries: [(rid, tokens, want)] — each request's next tokens and the
+        places among them whose logits are asked for. A request is admitted
+        at its first entry; `end` lists the requests that give their cache
+        blocks and state slot back after this step. The step goes the way a
+        generation step goes: the scheduler forms one batch (portions of
+        several tokens as prefill chunks, a request's single next token as a
+        decode row), the cache manager grows the block tables, and the same
+        forwards run. Returns fp32 logits [wanted, vocab] in the order of the
+        entries (None when nothing is wanted, or off the last stage)."""
+        batch, starts = self.scheduler.form_forced_batch(
+            [(rid, list(tokens)) for rid, tokens, _ in entries]
+        )
+        self.step_count += 1
+        want_of = {rid: list(want) for rid, _, want in entries}
+        rows = {}
+        with torch.inference_mode():
+            if batch.prefill_chunks:
+                flat, owners, t = [], [], 0
+                for c in batch.prefill_chunks:
+                    for k in want_of[c.req.rid]:
+                        flat.append(t + k)
+                        owners.append(c.req.rid)
+                    t += c.num_tokens
+                logits = self._prefill_group(batch.prefill_chunks, logits_at=flat)
+                if logits is not None:
+                    for i, rid in enumerate(owners):
+                        rows.setdefault(rid, []).append(logits[i])
+            if batch.decode_reqs:
+                logits = self._decode_one(batch.decode_reqs)
+                if logits is not None:
+                    for i, r in enumerate(batch.decode_reqs):
+                        if want_of[r.rid]:
+                            rows.setdefault(r.rid, []).append(logits[i].clone())
+        for c in batch.prefill_chunks:
+            c.req.num_prefilled_tokens = c.start + c.num_tokens
+        for r in batch.decode_reqs:
+            r.num_prefilled_tokens = r.prompt_len
+        for rid in end:
+            self.scheduler.finish_forced(rid)
+        out = [row for rid, _, _ in entries for row in rows.get(rid, [])]
+        if not out:
+            return None
+        return torch.stack(out).float()
 
     # -- convenience: synchronous generation (tests, chat CLI) --------------------------------
 

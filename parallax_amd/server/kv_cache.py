@@ -106,14 +106,23 @@ class MLAKVCache:
         dtype: torch.dtype = torch.bfloat16,
         index_dim: int = 0,
     ):
-        self.kv_lora_rank = kv_lora_rank
-        self.rope_dim = rope_dim
+        # kv_lora_rank / rope_dim may be per-layer sequences (stacks whose
+        # latent layers differ in size); scalars mean every layer is alike
+        ranks = list(kv_lora_rank) if isinstance(kv_lora_rank, (list, tuple)) \
+            else [kv_lora_rank] * num_layers
+        ropes = list(rope_dim) if isinstance(rope_dim, (list, tuple)) \
+            else [rope_dim] * num_layers
+        assert len(ranks) == len(ropes) == num_layers
+        self.kv_lora_rank = ranks[0] if ranks else 0
+        self.rope_dim = ropes[0] if ropes else 0
+        self.layer_ranks = ranks
+        self.layer_rope_dims = ropes
         self.block_size = block_size
         self.num_blocks = num_blocks
-        self.entry_dim = kv_lora_rank + rope_dim
+        self.entry_dim = self.kv_lora_rank + self.rope_dim
         self.caches: List[torch.Tensor] = [
-            torch.zeros((num_blocks, block_size, self.entry_dim), dtype=dtype, device=device)
-            for _ in range(num_layers)
+            torch.zeros((num_blocks, block_size, r + d), dtype=dtype, device=device)
+            for r, d in zip(ranks, ropes)
         ]
         # DSA (DeepSeek-V3.2): one indexer key per token per layer, shared
         # across indexer query heads (reference dsa_cache.py)
@@ -140,9 +149,12 @@ class MLAKVCache:
 
     @staticmethod
     def bytes_per_block(
-        num_layers: int, kv_lora_rank: int, rope_dim: int, block_size: int,
+        num_layers: int, kv_lora_rank, rope_dim, block_size: int,
         dtype: torch.dtype = torch.bfloat16, index_dim: int = 0,
     ) -> int:
+        if isinstance(kv_lora_rank, (list, tuple)):
+            width = sum(kv_lora_rank) + sum(rope_dim) + index_dim * num_layers
+            return block_size * width * dtype.itemsize
         return num_layers * block_size * (kv_lora_rank + rope_dim + index_dim) * dtype.itemsize
 
 
@@ -161,13 +173,21 @@ class LinearStateCache:
         dtype: torch.dtype = torch.bfloat16,
     ):
         self.num_slots = num_slots
+        # a list of shapes = one per layer (layers of unequal size)
+        conv_shapes = list(conv_state_shape) \
+            if conv_state_shape and isinstance(conv_state_shape[0], (list, tuple)) \
+            else [conv_state_shape] * num_layers
+        rec_shapes = list(recurrent_state_shape) \
+            if recurrent_state_shape and isinstance(recurrent_state_shape[0], (list, tuple)) \
+            else [recurrent_state_shape] * num_layers
+        assert len(conv_shapes) == len(rec_shapes) == num_layers
         self.conv_states: List[torch.Tensor] = [
-            torch.zeros((num_slots, *conv_state_shape), dtype=dtype, device=device)
-            for _ in range(num_layers)
+            torch.zeros((num_slots, *shape), dtype=dtype, device=device)
+            for shape in conv_shapes
         ]
         self.recurrent_states: List[torch.Tensor] = [
-            torch.zeros((num_slots, *recurrent_state_shape), dtype=torch.float32, device=device)
-            for _ in range(num_layers)
+            torch.zeros((num_slots, *shape), dtype=torch.float32, device=device)
+            for shape in rec_shapes
         ]
 
     def reset_slot(self, slot: int) -> None:

@@ -97,6 +97,10 @@ class InitialRequest(Request):
     # lazily-built constrained-decoding matcher (sampling_params.json_schema);
     # lives on the rank that samples, never serialized
     grammar: Optional[object] = field(default=None, repr=False, compare=False)
+    # teacher-forced replay: every token is given from outside (none is
+    # sampled), the "prompt" grows step by step and a step's single token
+    # runs through the decode path
+    forced: bool = False
 
     @property
     def prompt_len(self) -> int:
@@ -117,6 +121,12 @@ class InitialRequest(Request):
     @property
     def all_token_ids(self) -> List[int]:
         return self.prompt_token_ids + self.output_token_ids
+
+    def decode_input(self):
+        """(token fed to the next decode forward, its position)."""
+        if self.forced:
+            return self.prompt_token_ids[-1], self.prompt_len - 1
+        return self.output_token_ids[-1], self.total_len - 1
 
     def commit_new_token(self, token_id: int) -> None:
         if self.first_token_time is None:

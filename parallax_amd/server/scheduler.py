@@ -176,6 +176,55 @@ class Scheduler:
                 used += 1
         return used
 
+    # -- teacher-forced replay ------------------------------------------------------------
+
+    def form_forced_batch(self, entries) -> Tuple[ScheduledBatch, Dict[str, int]]:
+        """One iteration over tokens given from outside. entries: [(rid,
+        tokens)]. Unknown rids are admitted (blocks for the tokens brought, a
+        state slot where the stack has recurrent layers); known ones grow.
+        A single token of a request that already holds context becomes a
+        decode row, anything else a prefill chunk that starts where the
+        request stands. Returns the batch and each rid's start position."""
+        batch = ScheduledBatch()
+        starts: Dict[str, int] = {}
+        for rid, tokens in entries:
+            if not tokens:
+                raise ValueError(f"request {rid!r}: a step must bring tokens")
+            if rid in starts:
+                raise ValueError(f"request {rid!r} appears twice in one step")
+            req = self.running.get(rid)
+            if req is None:
+                if len(self.running) >= self.max_batch_size:
+                    raise RuntimeError(
+                        f"{len(self.running)} requests are live; the engine "
+                        f"was sized for {self.max_batch_size}")
+                req = InitialRequest(rid=rid, prompt_token_ids=list(tokens),
+                                     forced=True)
+                self.cache.allocate_request(rid, req.prompt_token_ids, 0)
+                req.status = RequestStatus.PREFILLING
+                self.running[rid] = req
+                start = 0
+            else:
+                if not req.forced:
+                    raise ValueError(f"request {rid!r} is not a replayed one")
+                start = req.prompt_len
+                req.prompt_token_ids.extend(tokens)
+                self.cache.append_tokens(rid, req.prompt_len)
+            starts[rid] = start
+            if len(tokens) == 1 and start > 0:
+                req.status = RequestStatus.DECODING
+                batch.decode_reqs.append(req)
+            else:
+                req.status = RequestStatus.PREFILLING
+                batch.prefill_chunks.append(PrefillChunk(req, start, len(tokens)))
+        return batch, starts
+
+    def finish_forced(self, rid: str) -> None:
+        req = self.running.pop(rid, None)
+        if req is None:
+            return
+        self.cache.free_request(rid, None)
+
     # -- step completion -----------------------------------------------------------
 
     def complete_prefill_chunk(self, chunk: PrefillChunk) -> None:

@@ -2,8 +2,11 @@
 
     PYTORCH_ROCM_ARCH=gfx950 python setup.py build_ext --inplace
 
-The built .so lands at parallax_amd/ops/_C.*.so (git-ignored; it travels to the
-GPU box with the gpurun snapshot).
+The built .so files land at parallax_amd/ops/_C.*.so (attention, GEMM, MoE,
+sampler kernels) and parallax_amd/ops/_mix.*.so (sequence mixers: fp32-residual
+layer norm, sliding-window latent attention, gated linear attention). Both are
+git-ignored; they travel to the GPU box with the gpurun snapshot.
+PARALLAX_EXT=_mix (or _C) builds one of them only.
 """
 
 import os
@@ -31,25 +34,49 @@ sources = [
 ]
 sources = [s for s in sources if os.path.exists(s)]
 
+HIP_FLAGS = [
+    "-O3",
+    "-std=c++17",
+    "--offload-arch=gfx950",
+]
+# hipcc turns plain float code into packed-fp32 instructions at -O3; the new
+# kernels keep every fp32 operation scalar
+MIX_HIP_FLAGS = HIP_FLAGS + ["-Xclang", "-target-feature", "-Xclang",
+                             "-packed-fp32-ops"]
+
+mix_sources = [
+    os.path.join(CSRC, "mix_bindings.cpp"),
+    os.path.join(CSRC, "layernorm.hip"),
+    os.path.join(CSRC, "latent_attention.hip"),
+    os.path.join(CSRC, "gla.hip"),
+]
+
+wanted = [x for x in os.environ.get("PARALLAX_EXT", "_C,_mix").split(",") if x]
+extensions = []
+if "_C" in wanted:
+    extensions.append(
+        CUDAExtension(
+            name="parallax_amd.ops._C",
+            sources=sources,
+            libraries=["hipblaslt"],
+            extra_compile_args={"cxx": ["-O3", "-std=c++17"], "nvcc": HIP_FLAGS},
+        )
+    )
+if "_mix" in wanted:
+    extensions.append(
+        CUDAExtension(
+            name="parallax_amd.ops._mix",
+            sources=mix_sources,
+            extra_compile_args={"cxx": ["-O3", "-std=c++17"],
+                                "nvcc": MIX_HIP_FLAGS},
+        )
+    )
+
 setup(
     name="parallax_amd_ext",
     entry_points={
         "console_scripts": ["parallax_amd = parallax_amd.cli:main"],
     },
-    ext_modules=[
-        CUDAExtension(
-            name="parallax_amd.ops._C",
-            sources=sources,
-            libraries=["hipblaslt"],
-            extra_compile_args={
-                "cxx": ["-O3", "-std=c++17"],
-                "nvcc": [
-                    "-O3",
-                    "-std=c++17",
-                    "--offload-arch=gfx950",
-                ],
-            },
-        )
-    ],
+    ext_modules=extensions,
     cmdclass={"build_ext": BuildExtension.with_options(use_ninja=True)},
 )
