@@ -1128,6 +1128,11 @@ class Engine:
             c.req.num_prefilled_tokens = c.start + c.num_tokens
         for r in batch.decode_reqs:
             r.num_prefilled_tokens = r.prompt_len
+        if self.device.type == "cuda":
+            # a replayed step has no sampled token to wait for; without this
+            # the host runs ahead and the next step rewrites the graph
+            # runner's pinned staging buffers under copies still in flight
+            torch.cuda.current_stream(self.device).synchronize()
         for rid in end:
             self.scheduler.finish_forced(rid)
         out = [row for rid, _, _ in entries for row in rows.get(rid, [])]
