@@ -151,6 +151,18 @@ class VurizenShardModel(nn.Module):
         return layers
 
     @property
+    def graph_safe(self) -> bool:
+        """Whether a decode forward can be captured into a hipGraph: the
+        per-expert loop that serves expert sizes outside the grouped-GEMM
+        kernel's tiling reads routing results on the host."""
+        W = self.cfg.hidden_size
+        return all(
+            layer.mlp is None
+            or (W % 32 == 0 and layer.mlp.intermediate_size % 64 == 0)
+            for layer in self.layers
+        )
+
+    @property
     def num_local_layers(self) -> int:
         return len(self.layers)
 
@@ -231,6 +243,8 @@ class VurizenShardModel(nn.Module):
         parts = local.split(".")
         layer: VurizenLayer = self.layers[int(parts[1])]
         key = ".".join(parts[2:])
+        if layer.mlp is None and key in ("norm2", "norm2.b", "ls2"):
+            return False  # a layer without feed-forward has no use for them
         if key in ("norm1", "norm2"):
             getattr(layer, key).weight.data.copy_(t)
         elif key in ("norm1.b", "norm2.b"):

@@ -440,6 +440,7 @@ def gelu_and_mul(x: torch.Tensor) -> torch.Tensor:
 # this kernel's simple 2-barrier structure; opt in for experiments.
 SKINNY_GEMM_MAX_M = int(os.environ.get("PARALLAX_SKINNY_GEMM_MAX_M", "0"))
 LT_GEMM = os.environ.get("PARALLAX_LT_GEMM", "1") != "0"
+_LT_REFUSED = set()  # (N, K) shapes hipBLASLt had no algorithm for
 
 
 def linear(
@@ -471,13 +472,24 @@ def linear(
         and weight.dtype == torch.bfloat16
         and x.is_contiguous()
         and weight.is_contiguous()
+        and weight.shape[0] % 8 == 0
+        and weight.shape[1] % 8 == 0
+        and (weight.shape[0], weight.shape[1]) not in _LT_REFUSED
     ):
         # tuned hipBLASLt: the default heuristic's decode-shape tile picks
         # are ~2.5x off the weight-streaming roofline (profiles/README.md);
         # first call per shape times the heuristic candidates (engine warmup,
         # outside graph capture) and later calls replay the winner
         ext = _require_ext("lt_linear")
-        y = ext.lt_linear(x, weight)
+        try:
+            y = ext.lt_linear(x, weight)
+        except RuntimeError as e:
+            # hipBLASLt offers no algorithm for some odd shapes: those go to
+            # torch's GEMM from now on (still a vendor product, never eager math)
+            if "hipblaslt" not in str(e):
+                raise
+            _LT_REFUSED.add((weight.shape[0], weight.shape[1]))
+            return torch.nn.functional.linear(x, weight, bias)
         return y if bias is None else y + bias
     return torch.nn.functional.linear(x, weight, bias)
 

@@ -255,7 +255,8 @@ class Engine:
         )
         self.sampler = Sampler(self.device, args.seed)
         self.graph_runner = None
-        if args.enable_graphs and self.device.type == "cuda":
+        if args.enable_graphs and self.device.type == "cuda" \
+                and getattr(self.model, "graph_safe", True):
             from .graph_runner import DecodeGraphRunner
 
             self.graph_runner = DecodeGraphRunner(

@@ -113,6 +113,10 @@ class DecodeGraphRunner:
         # block boundary or the batch composition changes
         self._cached_rids: List[str] = []
         self._cached_btlens: List[int] = []
+        # the table OBJECTS last copied: a request id that comes back after
+        # its request ended names a new table (other pages), and holding the
+        # old list keeps its identity from being recycled
+        self._cached_tables: List[List[int]] = []
 
     def _meta(self, bucket: int, ctx_bucket: Optional[int] = None) -> ForwardMeta:
         return ForwardMeta(
@@ -228,7 +232,11 @@ class DecodeGraphRunner:
         self.h_seq_lens[B:bucket] = 1
 
         btlens = [len(bt) for bt in block_tables]
-        same_batch = rids is not None and rids == self._cached_rids
+        same_batch = (
+            rids is not None and rids == self._cached_rids
+            and len(block_tables) == len(self._cached_tables)
+            and all(a is b for a, b in zip(block_tables, self._cached_tables))
+        )
         if same_batch:
             # steady-state decode: copy only rows whose table grew
             for i, bt in enumerate(block_tables):
@@ -248,6 +256,7 @@ class DecodeGraphRunner:
             )
         self._cached_rids = list(rids) if rids is not None else []
         self._cached_btlens = btlens
+        self._cached_tables = list(block_tables)
 
         if input_ids_dev is None:
             self.input_ids[:bucket].copy_(self.h_input_ids[:bucket],
