@@ -144,6 +144,143 @@ MODELS = {
 }
 
 
+# -- design comparison: Vurizen beside the closest existing family -------------------
+#
+# `--design-compare` leaves the headline workload alone and instead measures
+# prefill and decode throughput of a Vurizen stack (GLA + sliding-window latent
+# attention + grouped sigmoid MoE) and of a DeepSeek-V3-style stack (MLA +
+# the same router and experts) of EQUAL sizes, random weights, one GPU.
+
+DESIGN_SIZES = {
+    # width, layers, heads, nope, rot, vdim, rank, window, experts, top, ff, groups, keep
+    # (rank 512 / rot 64 everywhere: the only geometry the MLA decode kernel of
+    # the DeepSeek family is built for)
+    "s": dict(width=1024, layers=8, heads=8, nope=64, rot=64, vdim=64, rank=512,
+              window=1024, experts=16, top=2, ff=512, groups=4, keep=2, vocab=32000),
+    "m": dict(width=2048, layers=8, heads=16, nope=128, rot=64, vdim=128, rank=512,
+              window=4096, experts=32, top=4, ff=1024, groups=8, keep=4, vocab=32000),
+}
+
+
+def vurizen_config(z: dict) -> dict:
+    moe = {"kind": "moe", "expert": {"ff": z["ff"]},
+           "router": {"experts": z["experts"], "top": z["top"], "scale": 2.5,
+                      "groups": {"count": z["groups"], "keep": z["keep"]}}}
+
+    def latent(kv_from=None):
+        mx = {"heads": z["heads"], "dim": z["nope"], "rot_dim": z["rot"],
+              "vdim": z["vdim"], "kv_rank": z["rank"], "mask": {"size": z["window"]},
+              "scale": (z["nope"] + z["rot"]) ** -0.5,
+              "rot": {"dims": z["rot"], "base": 10000.0,
+                      "scaling": {"factor": 8.0, "original": 4096, "fast": 32.0,
+                                  "slow": 1.0}}}
+        if kv_from is not None:
+            mx["kv_from"] = kv_from
+        return {"type": "latent_attention", "mixer": mx, "mlp": moe}
+
+    gla = {"type": "gla", "mixer": {"heads": z["heads"], "dim": z["nope"],
+                                    "vdim": z["vdim"], "tau": 32.0}, "mlp": moe}
+    layers = []
+    for i in range(z["layers"]):   # gla, latent, latent reading it, latent, ...
+        k = i % 4
+        layers.append(gla if k == 0 else latent(i - 1 if k == 2 else None))
+    return {"architecture": "Vurizen", "layers": layers, "norm": {"eps": 1e-5},
+            "residual_mult": 1.0, "vocab": z["vocab"], "width": z["width"]}
+
+
+def deepseek_like_config(z: dict) -> dict:
+    return {
+        "architectures": ["DeepseekV3ForCausalLM"], "model_type": "deepseek_v3",
+        "vocab_size": z["vocab"], "hidden_size": z["width"],
+        "num_hidden_layers": z["layers"], "num_attention_heads": z["heads"],
+        "num_key_value_heads": z["heads"], "intermediate_size": z["ff"],
+        "moe_intermediate_size": z["ff"], "n_routed_experts": z["experts"],
+        "num_experts_per_tok": z["top"], "n_shared_experts": 0,
+        "n_group": z["groups"], "topk_group": z["keep"],
+        "routed_scaling_factor": 2.5, "norm_topk_prob": True,
+        "first_k_dense_replace": 0, "q_lora_rank": 0, "kv_lora_rank": z["rank"],
+        "qk_nope_head_dim": z["nope"], "qk_rope_head_dim": z["rot"],
+        "v_head_dim": z["vdim"], "rms_norm_eps": 1e-5, "rope_theta": 10000.0,
+        "max_position_embeddings": 16384, "tie_word_embeddings": False,
+        "torch_dtype": "bfloat16",
+    }
+
+
+def design_compare(args) -> None:
+    from parallax_amd.models.config import ModelConfig
+    from parallax_amd.server.engine import Engine, EngineArgs
+    from parallax_amd.server.sampling_params import SamplingParams
+
+    results = []
+    for size in args.design_sizes.split(","):
+        z = DESIGN_SIZES[size]
+        for design, cfg_dict in (("vurizen", vurizen_config(z)),
+                                 ("deepseek-like", deepseek_like_config(z))):
+            if args.design_only and design != args.design_only:
+                continue
+            cfg = ModelConfig.from_hf_config(cfg_dict)
+            B, P = args.design_batch, args.design_prompt
+            new = args.warmup + args.steps + 4
+            eargs = EngineArgs(
+                block_size=32, max_batch_size=B,
+                max_num_tokens_per_batch=B * P, prefill_chunk_size=B * P,
+                num_kv_blocks=B * ((P + new) // 32 + 2), enable_prefix_cache=False,
+                dtype=torch.bfloat16, max_model_len=P + new + 32, seed=0,
+            )
+            engine = Engine(cfg, eargs, random_weights=True)
+            engine.warmup_gemms([B * P, B])
+            g = torch.Generator().manual_seed(7)
+            sp = SamplingParams(temperature=1.0, max_new_tokens=new, ignore_eos=True)
+
+            def submit_all():
+                for _ in range(B):
+                    engine.submit(torch.randint(0, cfg.vocab_size, (P,),
+                                                generator=g).tolist(), sp)
+
+            def prefill_all():
+                while True:
+                    engine.step()
+                    run = engine.scheduler.running
+                    if run and all(r.prefill_done and r.num_output_tokens >= 1
+                                   for r in run.values()):
+                        return
+
+            # one untimed prefill (GEMM tuning, allocator), then a timed one
+            submit_all()
+            prefill_all()
+            for rid in list(engine.scheduler.running):
+                engine.abort(rid)
+            while engine.has_work:
+                engine.step()
+            submit_all()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            prefill_all()
+            torch.cuda.synchronize()
+            prefill_s = time.perf_counter() - t0
+            for _ in range(args.warmup):
+                engine.step()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(args.steps):
+                engine.step()
+            torch.cuda.synchronize()
+            decode_s = time.perf_counter() - t0
+            row = {
+                "design": design, "size": size, "batch": B, "prompt_len": P,
+                "prefill_tokens_per_s": round(B * P / prefill_s, 1),
+                "decode_tokens_per_s": round(B * args.steps / decode_s, 1),
+                "decode_ms_per_step": round(decode_s / args.steps * 1000, 3),
+                "dtype": "bf16", "data": "synthetic", "weights": "random",
+                "sizes": z,
+            }
+            results.append(row)
+            print(json.dumps(row), flush=True)
+            del engine
+            torch.cuda.empty_cache()
+    print(json.dumps({"metric": "design_compare", "rows": len(results)}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -177,7 +314,20 @@ def main():
                     help="override num_hidden_layers (reduced-layer single-GPU "
                          "runs of the PP=8 configs; headline runs use 0 = full)")
     ap.add_argument("--cpu", action="store_true", help="tiny CPU plumbing run")
+    ap.add_argument("--design-compare", action="store_true",
+                    help="instead of the headline workload: prefill and decode "
+                         "throughput of a Vurizen stack beside a DeepSeek-V3-"
+                         "style stack of equal sizes (one GPU, random weights)")
+    ap.add_argument("--design-sizes", default="s,m",
+                    help="comma list of " + ",".join(DESIGN_SIZES))
+    ap.add_argument("--design-batch", type=int, default=8)
+    ap.add_argument("--design-prompt", type=int, default=2048)
+    ap.add_argument("--design-only", default="",
+                    help="vurizen | deepseek-like (default: both)")
     args = ap.parse_args()
+    if args.design_compare:
+        design_compare(args)
+        return
 
     from parallax_amd.models.config import ModelConfig
     from parallax_amd.parallel.comm import CommContext, init_distributed

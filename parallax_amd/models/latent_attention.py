@@ -82,6 +82,7 @@ class LatentWindowAttention(nn.Module):
         out_lat = ops.latent_window_attention(
             q_lat.contiguous(), q_rot, cache, meta.block_tables,
             meta.token_seq(), meta.positions, self.window, self.scale,
+            max_seq_len=meta.max_seq_len,
         )
         attn = torch.einsum("thr,hvr->thv", out_lat, w_uv).to(x.dtype)
         return self.o_proj(attn.reshape(T, H * self.dv))

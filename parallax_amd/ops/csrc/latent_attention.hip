@@ -11,10 +11,14 @@
 //   latent_kv_store : RMS norm of the latent + rotation of the key part +
 //                     scatter into the paged cache, one kernel per layer.
 //   rope_rows       : rotation of the queries' rotated part into an fp32 buffer.
-//   latent_window_attention : one wave per (token, head), 64 keys per pass,
-//                     online softmax. A token sees keys j with
-//                     0 <= pos - j < window. Serves prompt portions and single
-//                     decoded tokens alike (a decode row is a portion of one).
+//   latent_window_attention : a workgroup per (token, group of heads, share of
+//                     the keys); 64 keys per wave and pass, online softmax,
+//                     every cache row converted once for all heads of the
+//                     group. A token sees keys j with 0 <= pos - j < window.
+//                     Prompt portions run one share per token; decode rows
+//                     split their window over several workgroups (fixed by
+//                     host-known sizes, so captured graphs stay valid) and a
+//                     small kernel joins the partial results.
 //
 // Angles are computed in fp32 from a per-layer frequency vector: pair
 // (i, i + rot_dims/2), a = pos * freq[i], cos and sin scaled by `mult`.
@@ -98,86 +102,251 @@ __global__ __launch_bounds__(256) void rope_rows_kernel(
 }
 
 #define LWA_WAVES 4
-#define LWA_MAX_RF 16  // latent features per lane: rank <= 64 * LWA_MAX_RF
 
-template <typename T, int RF>
+// 8 consecutive cache elements as floats (one 16-byte load for bf16, two for
+// float); p must be 16-byte aligned.
+template <typename T>
+DEVINL void load8(const T* p, float* v);
+template <>
+DEVINL void load8<bf16_t>(const bf16_t* p, float* v) {
+  const bf16x8 raw = load_bf16x8(p);
+#pragma unroll
+  for (int i = 0; i < 8; ++i) v[i] = bf16x8_get(raw, i);
+}
+template <>
+DEVINL void load8<float>(const float* p, float* v) {
+  const float4 a = *reinterpret_cast<const float4*>(p);
+  const float4 b = *reinterpret_cast<const float4*>(p + 4);
+  v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w;
+  v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+}
+
+// One workgroup = one token x one group of HB heads x one share of the keys.
+// All heads read the same cache rows, so a row is loaded and converted once
+// and used for HB heads. Score pass: a lane owns one key of a 64-key tile and
+// walks the row's features in 16-byte steps against the HB queries in LDS.
+// Value pass: a lane owns 8 consecutive latent features (x RC chunks of 512)
+// and walks the tile's keys. The window's tiles are dealt round-robin to the
+// 4 waves (x `splits` workgroups); each wave keeps its own online-softmax
+// state and they merge at the end (through `part` when splits > 1).
+// VEC: rows start 16-byte aligned and E is a multiple of 8 (else scalar loads).
+template <typename T, int HB, int RC, bool VEC>
 __global__ __launch_bounds__(256) void latent_window_attention_kernel(
-    float* __restrict__ out, const float* __restrict__ q_lat,
-    const float* __restrict__ q_rot, const T* __restrict__ cache,
-    const int* __restrict__ block_tables, int bt_stride,
-    const int* __restrict__ token_seq, const int* __restrict__ positions,
-    int H, int rank, int rot_w, int block_size, int window, float scale) {
+    float* __restrict__ out, float* __restrict__ part,
+    const float* __restrict__ q_lat, const float* __restrict__ q_rot,
+    const T* __restrict__ cache, const int* __restrict__ block_tables,
+    int bt_stride, const int* __restrict__ token_seq,
+    const int* __restrict__ positions, int H, int rank, int rot_w,
+    int block_size, int window, float scale, int splits) {
   extern __shared__ float lds[];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int64_t t = blockIdx.x;
-  int h = blockIdx.y * LWA_WAVES + wave;
-  const bool live = h < H;
-  if (!live) h = H - 1;
+  const int h0 = blockIdx.y * HB;
+  const int split = blockIdx.z;
   const int E = rank + rot_w;
-  const int Ep = (E + 1) & ~1;  // keeps the int64 row offsets 8-byte aligned
-  // per wave: q [Ep] | p [64] | row offsets [64] (as int64 -> 128 floats)
-  float* qs = lds + wave * (Ep + 64 + 128);
-  float* ps = qs + Ep;
-  int64_t* rows = reinterpret_cast<int64_t*>(ps + 64);
+  const int Ep = (E + 7) & ~7;
+  // LDS: q [HB][Ep] | per wave: p [HB][64], row offsets [64] (int64)
+  float* qs = lds;
+  float* ps = qs + HB * Ep + wave * (HB * 64 + 128);
+  int64_t* rows = reinterpret_cast<int64_t*>(ps + HB * 64);
 
-  const float* ql = q_lat + (t * H + h) * (int64_t)rank;
-  const float* qr = q_rot + (t * H + h) * (int64_t)rot_w;
-  for (int f = lane; f < rank; f += 64) qs[f] = ql[f];
-  for (int f = lane; f < rot_w; f += 64) qs[rank + f] = qr[f];
+  for (int idx = threadIdx.x; idx < HB * Ep; idx += 256) {
+    const int hh = idx / Ep, f = idx % Ep;
+    const int h = min(h0 + hh, H - 1);
+    float v = 0.f;
+    if (f < rank) v = q_lat[(t * H + h) * (int64_t)rank + f];
+    else if (f < E) v = q_rot[(t * H + h) * (int64_t)rot_w + (f - rank)];
+    qs[idx] = v;
+  }
 
   const int b = token_seq ? token_seq[t] : (int)t;
   const int pos = positions[t];
   const int lo = max(0, pos - window + 1);
   const int* bt = block_tables + (int64_t)b * bt_stride;
 
-  float m = -INFINITY, l = 0.f;
-  float acc[RF];
+  float m[HB], l[HB], acc[HB][RC][8];
 #pragma unroll
-  for (int k = 0; k < RF; ++k) acc[k] = 0.f;
+  for (int h = 0; h < HB; ++h) {
+    m[h] = -INFINITY;
+    l[h] = 0.f;
+#pragma unroll
+    for (int c = 0; c < RC; ++c)
+#pragma unroll
+      for (int i = 0; i < 8; ++i) acc[h][c][i] = 0.f;
+  }
   __syncthreads();
 
-  for (int j0 = lo; j0 <= pos; j0 += 64) {
+  const int stride = 64 * LWA_WAVES * splits;
+  for (int j0 = lo + 64 * (split * LWA_WAVES + wave); j0 <= pos; j0 += stride) {
     const int j = j0 + lane;
     const bool valid = j <= pos;
-    float s = -INFINITY;
     int64_t off = 0;
+    float s[HB];
+#pragma unroll
+    for (int h = 0; h < HB; ++h) s[h] = 0.f;
     if (valid) {
       off = ((int64_t)bt[j / block_size] * block_size + j % block_size) * E;
       const T* row = cache + off;
-      float d = 0.f;
-      for (int f = 0; f < E; ++f) d = fmaf(qs[f], ldf(row + f), d);
-      s = d * scale;
-    }
-    const float m_new = fmaxf(m, wave_reduce_max(s));
-    const float p = valid ? expf(s - m_new) : 0.f;
-    const float corr = expf(m - m_new);  // m = -inf at first: exp(-inf) = 0
-    l = l * corr + wave_reduce_sum(p);
-    m = m_new;
-    ps[lane] = p;
-    rows[lane] = off;
-    __syncthreads();
+      if (VEC) {
+        for (int f = 0; f < E; f += 8) {
+          float kv[8];
+          load8<T>(row + f, kv);
 #pragma unroll
-    for (int k = 0; k < RF; ++k) acc[k] *= corr;
+          for (int h = 0; h < HB; ++h) {
+            const float4 qa = *reinterpret_cast<const float4*>(qs + h * Ep + f);
+            const float4 qb = *reinterpret_cast<const float4*>(qs + h * Ep + f + 4);
+            s[h] = fmaf(qa.x, kv[0], s[h]);
+            s[h] = fmaf(qa.y, kv[1], s[h]);
+            s[h] = fmaf(qa.z, kv[2], s[h]);
+            s[h] = fmaf(qa.w, kv[3], s[h]);
+            s[h] = fmaf(qb.x, kv[4], s[h]);
+            s[h] = fmaf(qb.y, kv[5], s[h]);
+            s[h] = fmaf(qb.z, kv[6], s[h]);
+            s[h] = fmaf(qb.w, kv[7], s[h]);
+          }
+        }
+      } else {
+        for (int f = 0; f < E; ++f) {
+          const float kv = ldf(row + f);
+#pragma unroll
+          for (int h = 0; h < HB; ++h) s[h] = fmaf(qs[h * Ep + f], kv, s[h]);
+        }
+      }
+    }
+    float corr[HB];
+#pragma unroll
+    for (int h = 0; h < HB; ++h) {
+      const float sc = valid ? s[h] * scale : -INFINITY;
+      const float m_new = fmaxf(m[h], wave_reduce_max(sc));  // finite: key j0 is valid
+      const float p = valid ? expf(sc - m_new) : 0.f;
+      corr[h] = expf(m[h] - m_new);  // exp(-inf) = 0 on the first tile
+      l[h] = l[h] * corr[h] + wave_reduce_sum(p);
+      m[h] = m_new;
+      ps[h * 64 + lane] = p;
+    }
+    rows[lane] = off;
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+    for (int h = 0; h < HB; ++h)
+#pragma unroll
+      for (int c = 0; c < RC; ++c)
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc[h][c][i] *= corr[h];
     const int cnt = min(64, pos - j0 + 1);
     for (int jj = 0; jj < cnt; ++jj) {
-      const float pj = ps[jj];
       const T* row = cache + rows[jj];
 #pragma unroll
-      for (int k = 0; k < RF; ++k) {
-        const int f = lane + 64 * k;
-        if (f < rank) acc[k] = fmaf(pj, ldf(row + f), acc[k]);
+      for (int c = 0; c < RC; ++c) {
+        const int f = c * 512 + lane * 8;
+        if (f < rank) {
+          float cv[8];
+          if (VEC) {
+            load8<T>(row + f, cv);
+          } else {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) cv[i] = (f + i < rank) ? ldf(row + f + i) : 0.f;
+          }
+#pragma unroll
+          for (int h = 0; h < HB; ++h) {
+            const float pj = ps[h * 64 + jj];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) acc[h][c][i] = fmaf(pj, cv[i], acc[h][c][i]);
+          }
+        }
       }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  }
+
+  // ---- merge the 4 waves: common max, rescale, add up through LDS ----------------
+  __syncthreads();  // q and the per-wave regions are free from here on
+  float* wm = lds;                       // [4][HB]
+  float* wl = wm + LWA_WAVES * HB;       // [4][HB]
+  float* oacc = wl + LWA_WAVES * HB;     // [HB][rank_p], rank_p = RC * 512 cap
+  if (lane == 0) {
+#pragma unroll
+    for (int h = 0; h < HB; ++h) wm[wave * HB + h] = m[h];
+  }
+  __syncthreads();
+  float mg[HB], sc_w[HB];
+#pragma unroll
+  for (int h = 0; h < HB; ++h) {
+    float x = wm[h];
+    for (int w = 1; w < LWA_WAVES; ++w) x = fmaxf(x, wm[w * HB + h]);
+    mg[h] = x;
+    sc_w[h] = (m[h] == -INFINITY) ? 0.f : expf(m[h] - x);
+  }
+  if (lane == 0) {
+#pragma unroll
+    for (int h = 0; h < HB; ++h) wl[wave * HB + h] = l[h] * sc_w[h];
+  }
+  const int rank8 = (rank + 7) & ~7;
+  for (int w = 0; w < LWA_WAVES; ++w) {
+    if (wave == w) {
+#pragma unroll
+      for (int h = 0; h < HB; ++h)
+#pragma unroll
+        for (int c = 0; c < RC; ++c) {
+          const int f = c * 512 + lane * 8;
+          if (f < rank) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+              float* dst = oacc + h * rank8 + f + i;
+              const float v = acc[h][c][i] * sc_w[h];
+              *dst = (w == 0) ? v : *dst + v;
+            }
+          }
+        }
     }
     __syncthreads();
   }
-  if (live) {
-    const float inv = 1.0f / l;
-    float* o = out + (t * H + h) * (int64_t)rank;
-#pragma unroll
-    for (int k = 0; k < RF; ++k) {
-      const int f = lane + 64 * k;
-      if (f < rank) o[f] = acc[k] * inv;
+  // every thread: write the merged result
+  for (int idx = threadIdx.x; idx < HB * rank; idx += 256) {
+    const int hh = idx / rank, f = idx % rank;
+    const int h = h0 + hh;
+    if (h >= H) continue;
+    float lg = 0.f;
+    for (int w = 0; w < LWA_WAVES; ++w) lg += wl[w * HB + hh];
+    float mgh = wm[hh];
+    for (int w = 1; w < LWA_WAVES; ++w) mgh = fmaxf(mgh, wm[w * HB + hh]);
+    const float v = oacc[hh * rank8 + f];
+    if (splits == 1) {
+      out[(t * H + h) * (int64_t)rank + f] = v / lg;
+    } else {
+      float* pr = part + (((t * H + h) * (int64_t)splits + split) * (rank + 2));
+      pr[2 + f] = v;
+      if (f == 0) {
+        pr[0] = mgh;
+        pr[1] = lg;
+      }
     }
+  }
+}
+
+// out[t, h, :] from `splits` partial results [T, H, splits, 2 + rank]
+__global__ __launch_bounds__(256) void latent_window_reduce_kernel(
+    float* __restrict__ out, const float* __restrict__ part, int rank,
+    int splits) {
+  const int64_t th = blockIdx.x;
+  const float* pr = part + th * splits * (int64_t)(rank + 2);
+  float mg = -INFINITY;
+  for (int s = 0; s < splits; ++s) mg = fmaxf(mg, pr[s * (rank + 2)]);
+  float lg = 0.f;
+  for (int s = 0; s < splits; ++s) {
+    const float ms = pr[s * (rank + 2)];
+    lg += (ms == -INFINITY) ? 0.f : pr[s * (rank + 2) + 1] * expf(ms - mg);
+  }
+  for (int f = threadIdx.x; f < rank; f += 256) {
+    float v = 0.f;
+    for (int s = 0; s < splits; ++s) {
+      const float ms = pr[s * (rank + 2)];
+      if (ms != -INFINITY) v += pr[s * (rank + 2) + 2 + f] * expf(ms - mg);
+    }
+    out[th * rank + f] = v / lg;
   }
 }
 
@@ -218,42 +387,76 @@ extern "C" void launch_rope_rows(float* out, const void* q, int64_t tok_stride,
                        col0, freq, mult, rot_dims, positions, H, rot_w);
 }
 
+template <typename T, int HB, int RC>
+static void launch_lwa_hb(float* out, float* part, const float* q_lat,
+                          const float* q_rot, const void* cache,
+                          const int* block_tables, int bt_stride,
+                          const int* token_seq, const int* positions, int T_,
+                          int H, int rank, int rot_w, int block_size, int window,
+                          float scale, int splits, hipStream_t stream) {
+  const int E = rank + rot_w;
+  const int Ep = (E + 7) & ~7;
+  const int rank8 = (rank + 7) & ~7;
+  const size_t run = (size_t)HB * Ep + LWA_WAVES * (HB * 64 + 128);
+  const size_t merge = 2 * LWA_WAVES * HB + (size_t)HB * rank8;
+  const size_t shm = sizeof(float) * (run > merge ? run : merge);
+  const dim3 grid(T_, (H + HB - 1) / HB, splits);
+  const bool vec = (E % 8 == 0) && (sizeof(T) == 2 || E % 4 == 0);
+  if (vec)
+    hipLaunchKernelGGL((latent_window_attention_kernel<T, HB, RC, true>), grid,
+                       dim3(256), shm, stream, out, part, q_lat, q_rot,
+                       (const T*)cache, block_tables, bt_stride, token_seq,
+                       positions, H, rank, rot_w, block_size, window, scale,
+                       splits);
+  else
+    hipLaunchKernelGGL((latent_window_attention_kernel<T, HB, RC, false>), grid,
+                       dim3(256), shm, stream, out, part, q_lat, q_rot,
+                       (const T*)cache, block_tables, bt_stride, token_seq,
+                       positions, H, rank, rot_w, block_size, window, scale,
+                       splits);
+  if (splits > 1)
+    hipLaunchKernelGGL(latent_window_reduce_kernel, dim3(T_ * H), dim3(256), 0,
+                       stream, out, part, rank, splits);
+}
+
 template <typename T>
-static void launch_lwa_t(float* out, const float* q_lat, const float* q_rot,
-                         const void* cache, const int* block_tables,
-                         int bt_stride, const int* token_seq,
-                         const int* positions, int T_, int H, int rank,
-                         int rot_w, int block_size, int window, float scale,
-                         hipStream_t stream) {
-  const dim3 grid(T_, (H + LWA_WAVES - 1) / LWA_WAVES);
-  const size_t shm =
-      sizeof(float) * LWA_WAVES * (size_t)(((rank + rot_w + 1) & ~1) + 64 + 128);
-  const int rf = (rank + 63) / 64;
-#define LWA_LAUNCH(RF)                                                        \
-  hipLaunchKernelGGL((latent_window_attention_kernel<T, RF>), grid, dim3(256), \
-                     shm, stream, out, q_lat, q_rot, (const T*)cache,          \
-                     block_tables, bt_stride, token_seq, positions, H, rank,   \
-                     rot_w, block_size, window, scale)
-  if (rf <= 1) LWA_LAUNCH(1);
-  else if (rf <= 2) LWA_LAUNCH(2);
-  else if (rf <= 4) LWA_LAUNCH(4);
-  else if (rf <= 8) LWA_LAUNCH(8);
-  else LWA_LAUNCH(LWA_MAX_RF);
-#undef LWA_LAUNCH
+static void launch_lwa_t(float* out, float* part, const float* q_lat,
+                         const float* q_rot, const void* cache,
+                         const int* block_tables, int bt_stride,
+                         const int* token_seq, const int* positions, int T_,
+                         int H, int rank, int rot_w, int block_size, int window,
+                         float scale, int splits, hipStream_t stream) {
+#define LWA_ARGS                                                             \
+  out, part, q_lat, q_rot, cache, block_tables, bt_stride, token_seq,         \
+      positions, T_, H, rank, rot_w, block_size, window, scale, splits, stream
+  // heads per workgroup: 8 where the latent accumulators fit the registers
+  // (rank <= 512), 4 above; fewer when the model has fewer heads
+  if (rank <= 512) {
+    if (H >= 8) launch_lwa_hb<T, 8, 1>(LWA_ARGS);
+    else if (H >= 4) launch_lwa_hb<T, 4, 1>(LWA_ARGS);
+    else if (H >= 2) launch_lwa_hb<T, 2, 1>(LWA_ARGS);
+    else launch_lwa_hb<T, 1, 1>(LWA_ARGS);
+  } else {
+    if (H >= 4) launch_lwa_hb<T, 4, 2>(LWA_ARGS);
+    else if (H >= 2) launch_lwa_hb<T, 2, 2>(LWA_ARGS);
+    else launch_lwa_hb<T, 1, 2>(LWA_ARGS);
+  }
+#undef LWA_ARGS
 }
 
 extern "C" void launch_latent_window_attention(
-    float* out, const float* q_lat, const float* q_rot, const void* cache,
-    const int* block_tables, int bt_stride, const int* token_seq,
-    const int* positions, int T, int H, int rank, int rot_w, int block_size,
-    int window, float scale, int kind, hipStream_t stream) {
+    float* out, float* part, const float* q_lat, const float* q_rot,
+    const void* cache, const int* block_tables, int bt_stride,
+    const int* token_seq, const int* positions, int T, int H, int rank,
+    int rot_w, int block_size, int window, float scale, int splits, int kind,
+    hipStream_t stream) {
   if (T == 0) return;
   if (kind == 0)
-    launch_lwa_t<bf16_t>(out, q_lat, q_rot, cache, block_tables, bt_stride,
-                         token_seq, positions, T, H, rank, rot_w, block_size,
-                         window, scale, stream);
+    launch_lwa_t<bf16_t>(out, part, q_lat, q_rot, cache, block_tables,
+                         bt_stride, token_seq, positions, T, H, rank, rot_w,
+                         block_size, window, scale, splits, stream);
   else
-    launch_lwa_t<float>(out, q_lat, q_rot, cache, block_tables, bt_stride,
+    launch_lwa_t<float>(out, part, q_lat, q_rot, cache, block_tables, bt_stride,
                         token_seq, positions, T, H, rank, rot_w, block_size,
-                        window, scale, stream);
+                        window, scale, splits, stream);
 }

@@ -8,6 +8,8 @@
 
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
+
 extern "C" {
 void launch_add_layernorm(float*, const void*, int64_t, int, const void*, float,
                           const void*, const void*, float, void*, int, int, int,
@@ -18,10 +20,10 @@ void launch_latent_kv_store(const void*, int64_t, const void*, float,
                             hipStream_t);
 void launch_rope_rows(float*, const void*, int64_t, int64_t, int, const float*,
                       float, int, const int*, int, int, int, int, hipStream_t);
-void launch_latent_window_attention(float*, const float*, const float*,
+void launch_latent_window_attention(float*, float*, const float*, const float*,
                                     const void*, const int*, int, const int*,
                                     const int*, int, int, int, int, int, int,
-                                    float, int, hipStream_t);
+                                    float, int, int, hipStream_t);
 void launch_gla_recurrence(float*, const void*, const void*, const void*,
                            const void*, int64_t, int64_t, int64_t, int64_t,
                            const void*, float*, const int64_t*, const int*,
@@ -145,7 +147,7 @@ void latent_window_attention(torch::Tensor out, torch::Tensor q_lat,
                              torch::Tensor q_rot, torch::Tensor cache,
                              torch::Tensor block_tables, torch::Tensor token_seq,
                              torch::Tensor positions, int64_t window,
-                             double scale) {
+                             double scale, int64_t max_keys) {
   const int kind = kind_of(cache, "cache");
   CHECK_F32C(out);
   CHECK_F32C(q_lat);
@@ -169,12 +171,29 @@ void latent_window_attention(torch::Tensor out, torch::Tensor q_lat,
   } else {
     TORCH_CHECK(block_tables.size(0) >= T);
   }
+  // shares of the window per token: enough workgroups to fill the chip when
+  // there are few tokens (decode). Only host-known sizes enter, so a captured
+  // graph keeps its grid: max_keys is the longest context this launch can see.
+  const int64_t keys = std::max<int64_t>(1, std::min<int64_t>(window, max_keys));
+  const int64_t tiles_per_wg = 4;  // 64-key tiles, one per wave and round
+  const int hb = rank <= 512 ? 8 : 4;
+  const int64_t wgs = (int64_t)T * ((H + hb - 1) / hb);
+  int splits = 1;
+  if (wgs < 512) {
+    const int64_t by_keys = (keys + 64 * tiles_per_wg - 1) / (64 * tiles_per_wg);
+    const int64_t by_fill = (512 + wgs - 1) / wgs;
+    splits = (int)std::max<int64_t>(1, std::min<int64_t>({by_keys, by_fill, 32}));
+  }
+  torch::Tensor part;
+  if (splits > 1)
+    part = torch::empty({(int64_t)T, H, splits, rank + 2}, q_lat.options());
   launch_latent_window_attention(
-      out.data_ptr<float>(), q_lat.data_ptr<float>(), q_rot.data_ptr<float>(),
-      cache.data_ptr(), block_tables.data_ptr<int>(),
-      (int)block_tables.stride(0), has_seq ? token_seq.data_ptr<int>() : nullptr,
-      positions.data_ptr<int>(), T, H, rank, rot_w, (int)cache.size(1),
-      (int)window, (float)scale, kind, cur_stream());
+      out.data_ptr<float>(), splits > 1 ? part.data_ptr<float>() : nullptr,
+      q_lat.data_ptr<float>(), q_rot.data_ptr<float>(), cache.data_ptr(),
+      block_tables.data_ptr<int>(), (int)block_tables.stride(0),
+      has_seq ? token_seq.data_ptr<int>() : nullptr, positions.data_ptr<int>(),
+      T, H, rank, rot_w, (int)cache.size(1), (int)window, (float)scale, splits,
+      kind, cur_stream());
 }
 
 // q, k, z [T, H*dk] and v [T, H*dv] (row strides free), z_bias [H*dk],

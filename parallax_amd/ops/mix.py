@@ -92,11 +92,13 @@ def rope_rows(q, col0, rot_w, freq, mult, rot_dims, positions):
 
 
 def latent_window_attention(q_lat, q_rot, cache, block_tables, token_seq,
-                            positions, window, scale):
+                            positions, window, scale, max_seq_len=0):
     """Softmax attention of absorbed queries over the paged latent cache with
     a sliding window: token at position p sees keys p-window+1 .. p of its
     sequence. q_lat [T, H, rank] fp32, q_rot [T, H, rot_w] fp32, token_seq [T]
-    int32 (None: token i is sequence i). Returns fp32 [T, H, rank]."""
+    int32 (None: token i is sequence i). max_seq_len: the longest context in
+    the batch as the host knows it (0 = the block tables' capacity); it only
+    sizes the split of long windows over workgroups. Returns fp32 [T, H, rank]."""
     if not q_lat.is_cuda:
         return ref.latent_window_attention(q_lat, q_rot, cache, block_tables,
                                            token_seq, positions, window, scale)
@@ -105,6 +107,7 @@ def latent_window_attention(q_lat, q_rot, cache, block_tables, token_seq,
         out, q_lat, q_rot, cache, block_tables,
         token_seq if token_seq is not None
         else _empty(positions), positions, int(window), float(scale),
+        int(max_seq_len) or block_tables.shape[1] * cache.shape[1],
     )
     return out
 
