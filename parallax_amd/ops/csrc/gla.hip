@@ -8,8 +8,8 @@
 // portions, or decoded one token at a time, goes through the very same
 // operations in the same order. Parallelism comes from the state's columns:
 // o_t[j] only needs column j of S, so a thread owns (part of) one column in
-// registers for the whole portion. G lanes share a column when dk > 32 (each
-// holds 32 rows; their partial dot products meet through wave shuffles).
+// registers for the whole portion. G lanes share a column when dk > 16 (each
+// holds 16 rows; their partial dot products meet through wave shuffles).
 // q, k, the decay and v of 16 tokens at a time are staged in LDS by the whole
 // block, which also turns z into alpha once per (token, channel) and not once
 // per column.
@@ -21,7 +21,7 @@
 #include "seq_common.h"
 
 #define GLA_TC_MAX 16  // tokens staged per pass (fewer when dk is large)
-#define GLA_ROWS 32  // state rows per lane
+#define GLA_ROWS 16  // state rows per lane
 
 template <typename T>
 __global__ __launch_bounds__(256) void gla_recurrence_kernel(

@@ -210,7 +210,7 @@ void gla_recurrence(torch::Tensor o, torch::Tensor q, torch::Tensor k,
   const int H = state.size(1), dk = state.size(2), dv = state.size(3);
   const int T = o.size(0);
   TORCH_CHECK(o.size(1) == H && o.size(2) == dv);
-  TORCH_CHECK(dk <= 2048, "gla key dim above 2048 is not supported");
+  TORCH_CHECK(dk <= 1024, "gla key dim above 1024 is not supported");
   for (const torch::Tensor* t : {&q, &k, &z}) {
     TORCH_CHECK(t->is_cuda() && t->scalar_type() == q.scalar_type() &&
                 t->dim() == 2 && t->size(0) == T && t->size(1) == H * dk &&

@@ -26,7 +26,7 @@ def _tol(dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
-@pytest.mark.parametrize("W", [48, 256, 1000])
+@pytest.mark.parametrize("W", [48, 256, 1000, 4500])
 @pytest.mark.parametrize("y_fp32", [False, True])
 def test_add_layernorm(dtype, W, y_fp32):
     T = 7
