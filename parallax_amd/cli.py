@@ -5,6 +5,8 @@
   serve  — single-host serving: engine + OpenAI frontend in one process
            (PP over local GPUs via torch.distributed.run when --gpus > 1)
   chat   — minimal terminal chat client against any OpenAI endpoint
+  trace  — replay a JSON-lines token trace through the engine and write the
+           logits at the asked positions (same program as bin/trace_run)
 """
 
 from __future__ import annotations
@@ -287,6 +289,19 @@ def main(argv=None) -> None:
     pc.add_argument("--max-tokens", type=int, default=256)
     pc.set_defaults(fn=cmd_chat)
 
+    pt = sub.add_parser(
+        "trace", add_help=False,
+        help="replay a token trace (JSON lines on stdin) and write logits; "
+             "arguments as bin/trace_run (--model --dtype --out --max-tokens)")
+    pt.set_defaults(fn=None)
+
+    import sys as _sys
+
+    raw = list(_sys.argv[1:] if argv is None else argv)
+    if raw and raw[0] == "trace":
+        from .server.trace_replay import main as trace_main
+
+        raise SystemExit(trace_main(raw[1:]))
     args = p.parse_args(argv)
     args.fn(args)
 

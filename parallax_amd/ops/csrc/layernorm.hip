@@ -25,14 +25,25 @@ __global__ __launch_bounds__(256) void add_layernorm_kernel(
   float v[REG ? LN_NV : 1];
   float sum = 0.f;
   if (REG) {
+    // all loads first, unconditionally (index clamped), so they are in
+    // flight together instead of one dependent wait per element
+    float yv[LN_NV], sv[LN_NV];
+#pragma unroll
+    for (int k = 0; k < LN_NV; ++k) {
+      const int i = threadIdx.x + k * 256;
+      const int ic = i < W ? i : 0;
+      v[k] = x[ic];
+      yv[k] = yr ? ldf(yr + ic) : 0.f;
+      sv[k] = yr ? ldf(scale + ic) : 0.f;
+    }
 #pragma unroll
     for (int k = 0; k < LN_NV; ++k) {
       const int i = threadIdx.x + k * 256;
       float t = 0.f;
       if (i < W) {
-        t = x[i];
+        t = v[k];
         if (yr) {
-          t += mult * (ldf(scale + i) * ldf(yr + i));
+          t += mult * (sv[k] * yv[k]);
           x[i] = t;
         }
       }
@@ -67,10 +78,18 @@ __global__ __launch_bounds__(256) void add_layernorm_kernel(
   const float rstd = 1.0f / sqrtf(var + eps);
   TP* o = out + row * W;
   if (REG) {
+    float wv[LN_NV], bv[LN_NV];
 #pragma unroll
     for (int k = 0; k < LN_NV; ++k) {
       const int i = threadIdx.x + k * 256;
-      if (i < W) stf(o + i, (v[k] - mean) * rstd * ldf(w + i) + ldf(b + i));
+      const int ic = i < W ? i : 0;
+      wv[k] = ldf(w + ic);
+      bv[k] = ldf(b + ic);
+    }
+#pragma unroll
+    for (int k = 0; k < LN_NV; ++k) {
+      const int i = threadIdx.x + k * 256;
+      if (i < W) stf(o + i, (v[k] - mean) * rstd * wv[k] + bv[k]);
     }
   } else {
     for (int i = threadIdx.x; i < W; i += 256)

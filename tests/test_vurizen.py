@@ -387,3 +387,44 @@ def test_greedy_generation_through_the_scheduler(ckpt):
             seq.append(int(oracle.forward(cfg, w, seq)[-1].argmax()))
         assert got == seq[len(p):]
     assert eng.cache_manager.slot_allocator.num_free_slots == 4
+
+
+def test_trace_replay_program(ckpt, tmp_path):
+    """bin/trace_run: JSON lines in, 'done <step>' lines and <step>.f32 files
+    out; a step without wanted places writes no file; ended requests give
+    their pages and slots back."""
+    import json
+    import os
+    import subprocess
+    import sys
+
+    import numpy as np
+
+    cfg, w, path = ckpt
+    a, b = U.tokens(21, cfg["vocab"], 60), U.tokens(9, cfg["vocab"], 61)
+    steps = [
+        {"step": 0, "entries": [{"id": "a", "tokens": a[:16], "want": [0, 15]}], "end": []},
+        {"step": 1, "entries": [{"id": "a", "tokens": a[16:17], "want": []},
+                                {"id": "b", "tokens": b[:8], "want": [7]}], "end": []},
+        {"step": 2, "entries": [{"id": "b", "tokens": b[8:], "want": [0]},
+                                {"id": "a", "tokens": a[17:], "want": [3]}], "end": ["a", "b"]},
+    ]
+    repo = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    out = tmp_path / "logits"
+    p = subprocess.run(
+        [sys.executable, os.path.join(repo, "bin", "trace_run"), "--model", path,
+         "--dtype", "float32", "--out", str(out), "--max-tokens", "64", "--device", "cpu"],
+        input="\n".join(json.dumps(s) for s in steps) + "\n", capture_output=True,
+        text=True, timeout=300)
+    assert p.returncode == 0, p.stderr[-2000:]
+    assert [l for l in p.stdout.splitlines() if l.startswith("done")] == \
+        ["done 0", "done 1", "done 2"]
+    V = cfg["vocab"]
+    la, lb = oracle.forward(cfg, w, a), oracle.forward(cfg, w, b)
+    got0 = np.fromfile(out / "0.f32", dtype="<f4").reshape(-1, V)
+    got1 = np.fromfile(out / "1.f32", dtype="<f4").reshape(-1, V)
+    got2 = np.fromfile(out / "2.f32", dtype="<f4").reshape(-1, V)
+    assert got0.shape[0] == 2 and got1.shape[0] == 1 and got2.shape[0] == 2
+    want = torch.stack([la[0], la[15], lb[7], lb[8], la[20]])
+    got = torch.from_numpy(np.concatenate([got0, got1, got2]))
+    assert U.rel_err(got, want) < TOL
