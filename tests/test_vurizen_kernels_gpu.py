@@ -86,7 +86,8 @@ def test_latent_kv_store_and_rope_rows(dtype, rank, rot_w, rot_dims):
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("H,rank,rot_w,window", [(4, 96, 16, 23), (5, 72, 16, 7),
-                                                 (2, 520, 64, 300), (3, 32, 8, 1)])
+                                                 (2, 520, 64, 300), (3, 32, 8, 1),
+                                                 (3, 36, 6, 11)])
 def test_latent_window_attention(dtype, H, rank, rot_w, window):
     bs, nb = 8, 64
     E = rank + rot_w
