@@ -60,9 +60,12 @@ def test_mixed_batches(ckpt, dtype, graphs):
     eng = U.make_engine(path, device="cuda", dtype=dtype, pages=24, graphs=graphs)
     assert (eng.graph_runner is not None) == graphs
     got = U.run_schedule(eng, seqs, SCHEDULE)
+    alone = U.make_engine(path, device="cuda", dtype=dtype, pages=24)
     for name, toks in seqs.items():
         assert close(got[name], oracle.forward(cfg, w, toks), dtype), \
             (name, U.describe(got[name], oracle.forward(cfg, w, toks), TOL[dtype]))
+        whole = U.run_schedule(alone, {name: toks}, [[(name, len(toks))]])[name]
+        assert U.same_as_whole(got[name], whole), (name, U.describe(got[name], whole, 0.02))
     assert eng.cache_manager.num_free_blocks == 24
     assert eng.cache_manager.slot_allocator.num_free_slots == 4
 
@@ -72,12 +75,15 @@ def test_portions_decoding_and_reuse(ckpt, dtype):
     cfg, w, path = ckpt
     eng = U.make_engine(path, device="cuda", dtype=dtype, pages=20, max_requests=2,
                         graphs=dtype == torch.bfloat16)
+    alone = U.make_engine(path, device="cuda", dtype=dtype, pages=20)
     for k, cuts in enumerate([[150], [2] * 20 + [1] * 60, [3, 2, 7, 1, 1, 1, 33, 2, 5, 45],
                               [12] + [1] * 128]):
         toks = U.tokens(sum(cuts), cfg["vocab"], 40 + k)
         got = U.run_schedule(eng, {"r": toks}, [[("r", n)] for n in cuts])["r"]
         assert close(got, oracle.forward(cfg, w, toks), dtype), \
             (cuts[:3], U.describe(got, oracle.forward(cfg, w, toks), TOL[dtype]))
+        whole = U.run_schedule(alone, {"w": toks}, [[("w", len(toks))]])["w"]
+        assert U.same_as_whole(got, whole), (cuts[:3], U.describe(got, whole, 0.02))
         assert eng.cache_manager.num_free_blocks == 20
 
 

@@ -134,10 +134,20 @@ def close_in_bf16(got: torch.Tensor, want: torch.Tensor, tol: float) -> bool:
     two experts, which moves that position (and, through recurrent state, a
     little of what follows) by far more than rounding. Such rows are rare;
     a fault of the cache, state or batch hits most rows (and the float32
-    runs of the same kernels are held to rounding on every row). So: 85 rows
-    in 100 within tol and the median row well inside it."""
+    runs of the same kernels are held to rounding on every row). So: 70 rows
+    in 100 within tol and the median row well inside it. The sharper bf16
+    check is same_as_whole() below."""
     e = row_errs(got, want)
-    return bool((e < tol).double().mean() >= 0.85 and e.median() < tol / 3)
+    return bool((e < tol).double().mean() >= 0.7 and e.median() < tol / 3)
+
+
+def same_as_whole(got: torch.Tensor, whole: torch.Tensor, tol: float = 0.02) -> bool:
+    """A schedule's logits against the SAME engine dtype's logits for the
+    sequence run alone and whole: the arithmetic is the same up to GEMM tile
+    choices, so rows agree far inside bf16 rounding of the reference; 95 in
+    100 must (a router near-tie may still flip here and there)."""
+    e = row_errs(got, whole)
+    return bool((e < tol).double().mean() >= 0.95)
 
 
 def tokens(n: int, vocab: int, seed: int) -> List[int]:
