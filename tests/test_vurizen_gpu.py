@@ -36,6 +36,15 @@ def ckpt(tmp_path_factory):
     ]
     cfg = U.small_config(layers, width=64, vocab=131)
     w = oracle.random_weights(cfg, seed=3)
+    # corrections spaced wider than a sigmoid's range: which experts are
+    # chosen then never hangs on a near-tie that bf16 rounding could flip
+    # (data-dependent choices are held to rounding in the float32 runs and on
+    # the CPU engine); the weights of the chosen experts still follow the data
+    for k in list(w):
+        if k.endswith("mlp.correction"):
+            n = w[k].numel()
+            order = torch.randperm(n, generator=torch.Generator().manual_seed(n))
+            w[k] = (order.float() * 1.5).bfloat16().float()
     path = U.write_checkpoint(str(tmp_path_factory.mktemp("vzg")), cfg, w)
     return cfg, w, path
 

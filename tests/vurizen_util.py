@@ -130,15 +130,13 @@ def describe(got: torch.Tensor, want: torch.Tensor, tol: float) -> str:
 
 
 def close_in_bf16(got: torch.Tensor, want: torch.Tensor, tol: float) -> bool:
-    """bf16 rounding of a router's input now and then flips a near-tie between
-    two experts, which moves that position (and, through recurrent state, a
-    little of what follows) by far more than rounding. Such rows are rare;
-    a fault of the cache, state or batch hits most rows (and the float32
-    runs of the same kernels are held to rounding on every row). So: 70 rows
-    in 100 within tol and the median row well inside it. The sharper bf16
-    check is same_as_whole() below."""
+    """bf16 against the float64 reference: a sharp softmax or a router
+    near-tie makes single positions far more sensitive to rounding than the
+    rest, so: nine rows in ten within tol and the median row well inside it.
+    (The float32 runs of the same kernels are held to rounding on every row,
+    and same_as_whole() below is the sharper bf16 check.)"""
     e = row_errs(got, want)
-    return bool((e < tol).double().mean() >= 0.7 and e.median() < tol / 3)
+    return bool((e < tol).double().mean() >= 0.9 and e.median() < tol / 3)
 
 
 def same_as_whole(got: torch.Tensor, whole: torch.Tensor, tol: float = 0.02) -> bool:
