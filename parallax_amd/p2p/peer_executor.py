@@ -86,12 +86,18 @@ class PeerExecutor:
         if hasattr(self.model, "finalize_weights"):
             self.model.finalize_weights()
         self.model = self.model.to(device=self.device, dtype=dtype).eval()
-        self.model.rope_cache = self.model.rope_cache.float()
+        if getattr(self.model, "rope_cache", None) is not None:
+            self.model.rope_cache = self.model.rope_cache.float()
+        # what travels between peers: the activation dtype, or fp32 for
+        # stacks whose residual stream is fp32
+        self.hidden_dtype = getattr(self.model, "hidden_dtype", None) or dtype
 
-        self.is_mla = cfg.is_mla
+        self.is_mla = cfg.is_mla or cfg.layer_specs is not None
         if self.is_mla:
+            latent_dims = cfg.latent_cache_dims(start_layer, end_layer)
             self.kv_cache = MLAKVCache(
-                end_layer - start_layer, cfg.kv_lora_rank, cfg.qk_rope_head_dim,
+                len(latent_dims), [r for r, _ in latent_dims],
+                [d for _, d in latent_dims],
                 block_size, num_kv_blocks, self.device,
                 dtype if dtype != torch.float32 else torch.float32,
                 index_dim=cfg.index_head_dim if cfg.is_dsa else 0,
@@ -109,20 +115,14 @@ class PeerExecutor:
         if cfg.has_linear_layers:
             from ..server.kv_cache import LinearStateCache
 
-            local_types = [cfg.layer_type(g) for g in range(start_layer, end_layer)]
-            n_linear = sum(1 for t in local_types if t == "linear_attention")
-            conv_dim = (
-                2 * cfg.linear_num_key_heads * cfg.linear_key_head_dim
-                + cfg.linear_num_value_heads * cfg.linear_value_head_dim
-            )
+            shapes = cfg.linear_state_shapes(start_layer, end_layer)
+            if not shapes:  # no linear layer on this peer: one dummy entry
+                shapes = cfg.linear_state_shapes(0, cfg.num_layers)[:1]
             num_linear_slots = 64
             self.linear_cache = LinearStateCache(
-                max(1, n_linear),
-                conv_state_shape=(conv_dim, cfg.linear_conv_kernel_dim - 1),
-                recurrent_state_shape=(
-                    cfg.linear_num_value_heads, cfg.linear_key_head_dim,
-                    cfg.linear_value_head_dim,
-                ),
+                len(shapes),
+                conv_state_shape=[c for c, _ in shapes],
+                recurrent_state_shape=[r for _, r in shapes],
                 num_slots=num_linear_slots + 1,
                 device=self.device,
                 dtype=dtype if dtype != torch.float32 else torch.float32,
@@ -134,6 +134,8 @@ class PeerExecutor:
             enable_prefix_cache=self.is_head and not cfg.has_linear_layers,
             num_linear_slots=num_linear_slots,
         )
+        if self.linear_cache is not None:
+            self.cache_manager.on_slot_allocated = self.linear_cache.reset_slot
         self.scheduler = (
             Scheduler(self.cache_manager, eos_token_ids=cfg.eos_token_ids)
             if self.is_head else None
@@ -263,7 +265,7 @@ class PeerExecutor:
             chunks = batch.prefill_chunks
             meta, input_ids, _ = self._head_prefill_meta(chunks)
             with torch.inference_mode():
-                hidden = self.model.embed(input_ids).to(self.dtype)
+                hidden = self.model.embed(input_ids).to(self.hidden_dtype)
                 hidden = self.model(hidden, meta)
             packets = []
             t = 0
@@ -285,7 +287,7 @@ class PeerExecutor:
             reqs = batch.decode_reqs
             meta, input_ids = self._head_decode_meta(reqs)
             with torch.inference_mode():
-                hidden = self.model.embed(input_ids).to(self.dtype)
+                hidden = self.model.embed(input_ids).to(self.hidden_dtype)
                 hidden = self.model(hidden, meta)
             packets = []
             for i, r in enumerate(reqs):
@@ -372,7 +374,7 @@ class PeerExecutor:
             btabs.append(state.block_table)
             seq_lens.append(total)
             qlens.append(p.num_new_tokens)
-            hiddens.append(p.hidden_states.to(self.device, self.dtype))
+            hiddens.append(p.hidden_states.to(self.device, self.hidden_dtype))
             if self.is_last and p.sampling_params is not None:
                 ctx = self._sampling_ctx.setdefault(
                     p.rid, (p.sampling_params, [], [])

@@ -428,3 +428,84 @@ def test_trace_replay_program(ckpt, tmp_path):
     want = torch.stack([la[0], la[15], lb[7], lb[8], la[20]])
     got = torch.from_numpy(np.concatenate([got0, got1, got2]))
     assert U.rel_err(got, want) < TOL
+
+
+def test_two_peer_pipeline_greedy(ckpt):
+    """The packet-driven multi-host path: two peers split the stack (the fp32
+    residual travels between them), greedy tokens equal the reference's."""
+    from parallax_amd.p2p.peer_executor import PeerExecutor
+    from parallax_amd.p2p.transport import LoopbackTransport
+
+    cfg, w, path = ckpt
+    mc = ModelConfig.from_pretrained(path)
+    registry, peers = {}, []
+    # layer 2 reads layer 0's cache rows, so the cut comes after it
+    for pid, (s, e) in zip(["p0", "p1"], [(0, 3), (3, 5)]):
+        peers.append(PeerExecutor(mc, s, e, pid, LoopbackTransport(pid, registry),
+                                  dtype=torch.float32, num_kv_blocks=64, block_size=8,
+                                  model_path=path))
+    head = peers[0]
+    prompts = [U.tokens(19, cfg["vocab"], 70), U.tokens(4, cfg["vocab"], 71)]
+    sp = SamplingParams(temperature=0.0, max_new_tokens=6, ignore_eos=True)
+    rids = [head.submit(p, sp, ["p0", "p1"]) for p in prompts]
+    outputs, done = {r: [] for r in rids}, set()
+    for _ in range(2000):
+        for px in peers:
+            px.step(recv_timeout=0.001)
+        for out in head.drain_outputs():
+            outputs[out.rid].append(out.token_id)
+            if out.finished:
+                done.add(out.rid)
+        if len(done) == len(rids):
+            break
+    for p, rid in zip(prompts, rids):
+        seq = list(p)
+        for _ in range(6):
+            seq.append(int(oracle.forward(cfg, w, seq)[-1].argmax()))
+        assert outputs[rid] == seq[len(p):]
+    with pytest.raises(ValueError):   # a cut that separates a layer from the cache it reads
+        PeerExecutor(mc, 1, 3, "bad", LoopbackTransport("bad", registry),
+                     dtype=torch.float32, num_kv_blocks=8, block_size=8)
+
+
+def _pp_worker(rank, world, port, path, prompts, out_file):
+    import os
+
+    os.environ.update(MASTER_ADDR="127.0.0.1", MASTER_PORT=str(port),
+                      RANK=str(rank), WORLD_SIZE=str(world))
+    import torch.distributed as dist
+
+    from parallax_amd.parallel.comm import init_distributed
+    from parallax_amd.server.engine import Engine, EngineArgs
+
+    comm = init_distributed(pp_size=world, tp_size=1, backend="gloo",
+                            device=torch.device("cpu"))
+    eng = Engine(ModelConfig.from_pretrained(path),
+                 EngineArgs(block_size=8, num_kv_blocks=64, max_batch_size=4,
+                            dtype=torch.float32, micro_batches=2,
+                            enable_prefix_cache=False, max_model_len=512),
+                 comm=comm, model_path=path)
+    sp = [SamplingParams(temperature=0.0, max_new_tokens=5, ignore_eos=True)] * len(prompts)
+    outs = list(eng.generate(prompts, sp).values())
+    if rank == 0:
+        torch.save(outs, out_file)
+    dist.barrier()
+    dist.destroy_process_group()
+
+
+def test_pipeline_stages_over_gloo(ckpt, tmp_path):
+    """Two pipeline stages in two processes (gloo): the fp32 residual crosses
+    the stage boundary, greedy tokens equal the reference's."""
+    import torch.multiprocessing as mp
+
+    cfg, w, path = ckpt
+    prompts = [U.tokens(13, cfg["vocab"], 80), U.tokens(3, cfg["vocab"], 81),
+               U.tokens(26, cfg["vocab"], 82)]
+    out_file = str(tmp_path / "pp2.pt")
+    mp.spawn(_pp_worker, args=(2, 29671, path, prompts, out_file), nprocs=2, join=True)
+    got = torch.load(out_file)
+    for p, toks in zip(prompts, got):
+        seq = list(p)
+        for _ in range(5):
+            seq.append(int(oracle.forward(cfg, w, seq)[-1].argmax()))
+        assert toks == seq[len(p):]

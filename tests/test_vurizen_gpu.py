@@ -138,6 +138,9 @@ def test_greedy_generation_bf16_through_graphs(ckpt):
     the reference's best token or within rounding of it."""
     cfg, w, path = ckpt
     eng = U.make_engine(path, device="cuda", dtype=torch.bfloat16, graphs=True)
+    eng.warmup_serving()   # what `serve` does at start: GEMM picks, every decode graph
+    assert len(eng.graph_runner._graphs) == \
+        len(eng.graph_runner.buckets) * len(eng.graph_runner.ctx_buckets)
     prompts = [U.tokens(29, cfg["vocab"], 21), U.tokens(3, cfg["vocab"], 22),
                U.tokens(64, cfg["vocab"], 23)]
     sp = [SamplingParams(temperature=0.0, max_new_tokens=24, ignore_eos=True)] * 3
