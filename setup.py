@@ -34,15 +34,15 @@ sources = [
 ]
 sources = [s for s in sources if os.path.exists(s)]
 
+# hipcc -O3 turns plain float code into packed-fp32 instructions; every kernel
+# here keeps its fp32 operations scalar (-packed-fp32-ops)
 HIP_FLAGS = [
     "-O3",
     "-std=c++17",
     "--offload-arch=gfx950",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
 ]
-# hipcc turns plain float code into packed-fp32 instructions at -O3; the new
-# kernels keep every fp32 operation scalar
-MIX_HIP_FLAGS = HIP_FLAGS + ["-Xclang", "-target-feature", "-Xclang",
-                             "-packed-fp32-ops"]
+MIX_HIP_FLAGS = HIP_FLAGS
 
 mix_sources = [
     os.path.join(CSRC, "mix_bindings.cpp"),
