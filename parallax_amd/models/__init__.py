@@ -17,3 +17,4 @@ from . import qwen3_5  # noqa: F401
 from . import minimax  # noqa: F401
 from . import minimax_m3  # noqa: F401
 from . import vurizen  # noqa: F401
+from . import sogidra  # noqa: F401

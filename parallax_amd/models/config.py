@@ -86,7 +86,7 @@ class ModelConfig:
     linear_value_head_dim: int = 0
     linear_conv_kernel_dim: int = 4
 
-    # -- per-layer stacks (vurizen): every layer carries its own mixer and
+    # -- per-layer stacks (vurizen, sogidra): every layer carries its own mixer and
     # feed-forward description; the flat fields above hold the first layer's
     # values only so that sizing helpers have something to read ----------------
     layer_specs: Optional[List[Dict[str, Any]]] = None
@@ -109,19 +109,47 @@ class ModelConfig:
     # -- cache geometry per local layer (the engine sizes its pools from these) --
 
     def latent_cache_dims(self, start: int, end: int) -> List[tuple]:
-        """(latent rank, rotated-key width) of every layer in [start, end) that
-        OWNS a compressed-latent cache entry. Layers that read another layer's
-        entry (vurizen `kv_from`) and non-latent layers are left out."""
+        """Row geometry of every layer in [start, end) that OWNS a row-per-
+        token cache entry, as (first part, second part) widths: (latent rank,
+        rotated-key width) for compressed-latent layers, (key width, value
+        width) over all key/value heads for the row-attention mixers. Layers
+        that read another layer's entry (`kv_from`) and layers without a
+        paged cache are left out."""
         if self.layer_specs is not None:
-            return [
-                (int(sp["mixer"]["kv_rank"]), int(sp["mixer"]["rot_dim"]))
-                for sp in self.layer_specs[start:end]
-                if sp["type"] == "latent_attention"
-                and sp["mixer"].get("kv_from") is None
-            ]
+            dims = []
+            for sp in self.layer_specs[start:end]:
+                mx = sp["mixer"]
+                if mx.get("kv_from") is not None:
+                    continue
+                if sp["type"] == "latent_attention":
+                    dims.append((int(mx["kv_rank"]), int(mx["rot_dim"])))
+                elif sp["type"] == "attention":      # two score maps per head
+                    g = int(mx["kv_heads"])
+                    dims.append((g * 2 * int(mx["dim"]), g * int(mx["vdim"])))
+                elif sp["type"] == "attention_2":    # values = unnormed keys
+                    g = int(mx["kv_heads"])
+                    dims.append((g * int(mx["dim"]), g * int(mx["dim"])))
+            return dims
         if not self.is_mla:
             return []
         return [(self.kv_lora_rank, self.qk_rope_head_dim)] * (end - start)
+
+    def pooled_cache_blocks(self, start: int, end: int) -> List[int]:
+        """For every cache-owning layer of latent_cache_dims(start, end): the
+        number of tokens whose mean row the layer also keeps (pooled blocks
+        seen beyond a sliding window), 0 for layers that keep none."""
+        if self.layer_specs is None:
+            return [0] * len(self.latent_cache_dims(start, end))
+        out = []
+        for sp in self.layer_specs[start:end]:
+            mx = sp["mixer"]
+            if mx.get("kv_from") is not None:
+                continue
+            if sp["type"] in ("latent_attention", "attention"):
+                out.append(0)
+            elif sp["type"] == "attention_2":
+                out.append(int((mx.get("mask") or {}).get("pool", 0)))
+        return out
 
     def linear_state_shapes(self, start: int, end: int) -> List[tuple]:
         """(conv-state shape, recurrent-state shape) of every linear-attention
@@ -177,18 +205,26 @@ class ModelConfig:
     def from_layer_list_config(cls, cfg: Dict[str, Any]) -> "ModelConfig":
         """Configs that describe the stack as a list of layers
         ({"architecture": ..., "layers": [{"type", "mixer", "mlp"}, ...],
-        "norm": {"eps"}, "residual_mult", "vocab", "width"})."""
+        "norm": {"eps"}, "vocab", "width", ...}). Mixer types: 'gla',
+        'latent_attention' (vurizen); 'attention' (differential softmax
+        attention), 'attention_2' (sliding window with pooled blocks)
+        (sogidra). Feed-forward kinds: 'moe' (default), 'dense'."""
         layers = cfg["layers"]
-        kinds = {"gla": "linear_attention", "latent_attention": "latent_attention"}
+        kinds = {"gla": "linear_attention", "latent_attention": "latent_attention",
+                 "attention": "diff_attention",
+                 "attention_2": "pooled_window_attention"}
         for sp in layers:
             if sp["type"] not in kinds:
                 raise ValueError(f"unknown layer type {sp['type']!r}")
             mlp = sp.get("mlp")
-            if mlp is not None and mlp.get("kind", "moe") != "moe":
+            if mlp is not None and mlp.get("kind", "moe") not in ("moe", "dense"):
                 raise ValueError(f"unknown feed-forward kind {mlp.get('kind')!r}")
         latent = [sp["mixer"] for sp in layers if sp["type"] == "latent_attention"]
         linear = [sp["mixer"] for sp in layers if sp["type"] == "gla"]
-        moes = [sp["mlp"] for sp in layers if sp.get("mlp") is not None]
+        windowed = [sp["mixer"] for sp in layers if sp["type"] == "attention_2"]
+        mlps = [sp["mlp"] for sp in layers if sp.get("mlp") is not None]
+        moes = [m for m in mlps if m.get("kind", "moe") == "moe"]
+        dense = [m for m in mlps if m.get("kind", "moe") == "dense"]
         first = layers[0]["mixer"]
         mc = cls(
             architecture=cfg["architecture"],
@@ -197,7 +233,7 @@ class ModelConfig:
             hidden_size=int(cfg["width"]),
             num_layers=len(layers),
             num_heads=int(first["heads"]),
-            num_kv_heads=int(first["heads"]),
+            num_kv_heads=int(first.get("kv_heads", first["heads"])),
             head_dim=int(first["dim"]),
             rms_norm_eps=float(cfg["norm"]["eps"]),
             max_position_embeddings=int(cfg.get("max_positions", 1 << 20)),
@@ -215,11 +251,15 @@ class ModelConfig:
             mc.qk_rope_head_dim = int(latent[0]["rot_dim"])
             mc.v_head_dim = int(latent[0]["vdim"])
             mc.sliding_window = int(latent[0]["mask"]["size"])
+        if windowed:
+            mc.sliding_window = int(windowed[0]["mask"]["size"])
         if linear:
             mc.linear_num_key_heads = mc.linear_num_value_heads = int(linear[0]["heads"])
             mc.linear_key_head_dim = int(linear[0]["dim"])
             mc.linear_value_head_dim = int(linear[0]["vdim"])
             mc.linear_conv_kernel_dim = 1
+        if dense:
+            mc.intermediate_size = int(dense[0]["ff"])
         if moes:
             r = moes[0]["router"]
             mc.num_experts = int(r["experts"])

@@ -651,5 +651,10 @@ from .mix import (  # noqa: E402,F401
     has_mix_extension,
     latent_kv_store,
     latent_window_attention,
+    pool_cache_update,
+    qkv_store,
     rope_rows,
+    row_attention,
+    sandwich_rmsnorm,
+    xielu,
 )

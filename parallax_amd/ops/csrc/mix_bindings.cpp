@@ -1,6 +1,7 @@
 // Python bindings of the sequence-mixer kernels (extension parallax_amd.ops._mix):
 // fp32-residual layer norm, sliding-window latent attention, gated linear
-// attention. Every entry point checks shapes and types on the host before a
+// attention, sandwich RMS norm with depth averaging, row-cache attention
+// (differential / pooled sliding window), xIELU. Every entry point checks shapes and types on the host before a
 // launch; activation tensors are bf16 or float32 (one template instance each).
 
 #include <ATen/hip/HIPContext.h>
@@ -31,6 +32,24 @@ void launch_gla_recurrence(float*, const void*, const void*, const void*,
                            hipStream_t);
 void launch_gated_rmsnorm(void*, const float*, const void*, int64_t,
                           const void*, float, int, int, int, int, hipStream_t);
+void launch_sandwich_rmsnorm(float*, const void*, int64_t, int, const void*,
+                             float*, int64_t, int, const float*, const void*,
+                             float, float, void*, const void*, const int*, int,
+                             int, int, hipStream_t);
+void launch_xielu(void*, const void*, int64_t, float, float, int, hipStream_t);
+void launch_qkv_store(float*, const void*, int64_t, const void*, int64_t,
+                      const void*, int64_t, const int*, const int64_t*, void*,
+                      int, int, int, int, float, float, int, int, int,
+                      hipStream_t);
+void launch_pool_cache_update(const void*, float*, const int*, int, const int*,
+                              const int*, const int64_t*, int, int, int, int,
+                              int, int, hipStream_t);
+int row_attention_heads_per_group(int);
+void launch_row_attention(void*, float*, const float*, const void*,
+                          const float*, const int*, int, const int*, const int*,
+                          int, int, int, int, int, int, int, int, int, int,
+                          float, float, float, float, float, int, int,
+                          hipStream_t);
 }
 
 static hipStream_t cur_stream() {
@@ -258,6 +277,226 @@ void gated_rmsnorm(torch::Tensor out, torch::Tensor o, torch::Tensor gate,
                        dv, kind, cur_stream());
 }
 
+// x [T, W] fp32 (in place); y [T, W] (row stride free) + w_branch [W] or
+// empty; hist [n_max, T, W] fp32 or empty; dwa [n_hist] fp32 or empty; w_next
+// [W] + out [T, W] or empty; add_table [N, W] + add_index [T] int32 or empty
+void sandwich_rmsnorm(torch::Tensor x, torch::Tensor y, torch::Tensor w_branch,
+                      torch::Tensor hist, int64_t n_hist, torch::Tensor dwa,
+                      torch::Tensor w_next, double eps, double offset,
+                      torch::Tensor out, torch::Tensor add_table,
+                      torch::Tensor add_index) {
+  CHECK_F32C(x);
+  TORCH_CHECK(x.dim() == 2);
+  const int rows = x.size(0), W = x.size(1);
+  const bool has_y = y.numel() > 0, has_n = w_next.numel() > 0;
+  const bool has_h = hist.numel() > 0, has_d = dwa.numel() > 0;
+  const bool has_t = add_table.numel() > 0;
+  int y_kind = 1, p_kind = -1;
+  int64_t y_stride = 0;
+  auto param = [&](const torch::Tensor& t, const char* what) {
+    const int k = kind_of(t, what);
+    TORCH_CHECK(p_kind < 0 || k == p_kind, "parameter types differ");
+    p_kind = k;
+  };
+  if (has_y) {
+    y_kind = kind_of(y, "y");
+    TORCH_CHECK(y.dim() == 2 && y.size(0) == rows && y.size(1) == W &&
+                y.stride(1) == 1);
+    y_stride = y.stride(0);
+    param(w_branch, "w_branch");
+    TORCH_CHECK(w_branch.numel() == W && w_branch.is_contiguous());
+  }
+  if (has_n) {
+    param(w_next, "w_next");
+    TORCH_CHECK(w_next.numel() == W && w_next.is_contiguous());
+    TORCH_CHECK(out.is_cuda() && out.scalar_type() == w_next.scalar_type() &&
+                out.is_contiguous() && out.dim() == 2 && out.size(0) == rows &&
+                out.size(1) == W);
+  }
+  if (has_t) {
+    param(add_table, "add_table");
+    TORCH_CHECK(add_table.dim() == 2 && add_table.size(1) == W &&
+                add_table.is_contiguous());
+    CHECK_I32(add_index);
+    TORCH_CHECK(add_index.numel() == rows);
+  }
+  if (has_h) {
+    CHECK_F32C(hist);
+    TORCH_CHECK(hist.dim() == 3 && hist.size(1) == rows && hist.size(2) == W);
+    TORCH_CHECK(n_hist >= 1 && n_hist <= hist.size(0));
+  }
+  if (has_d) {
+    CHECK_F32C(dwa);
+    TORCH_CHECK(has_h && dwa.numel() == n_hist);
+  }
+  if (p_kind < 0) p_kind = 1;
+  launch_sandwich_rmsnorm(
+      x.data_ptr<float>(), has_y ? y.data_ptr() : nullptr, y_stride, y_kind,
+      has_y ? w_branch.data_ptr() : nullptr,
+      has_h ? hist.data_ptr<float>() : nullptr, (int64_t)rows * W, (int)n_hist,
+      has_d ? dwa.data_ptr<float>() : nullptr,
+      has_n ? w_next.data_ptr() : nullptr, (float)eps, (float)offset,
+      has_n ? out.data_ptr() : nullptr, has_t ? add_table.data_ptr() : nullptr,
+      has_t ? add_index.data_ptr<int>() : nullptr, p_kind, rows, W,
+      cur_stream());
+}
+
+void xielu(torch::Tensor out, torch::Tensor x, double a_pos, double a_neg) {
+  const int kind = kind_of(x, "x");
+  TORCH_CHECK(x.is_contiguous() && out.is_cuda() && out.is_contiguous() &&
+              out.scalar_type() == x.scalar_type() && out.numel() == x.numel());
+  launch_xielu(out.data_ptr(), x.data_ptr(), x.numel(), (float)a_pos,
+               (float)a_neg, kind, cur_stream());
+}
+
+// q [T, wq], k [T, wk] or empty, v [T, wv] or empty (values = k) — row strides
+// free; q_out [T, wq] fp32; cache [blocks, block, wk + wv]
+void qkv_store(torch::Tensor q_out, torch::Tensor q, torch::Tensor k,
+               torch::Tensor v, torch::Tensor positions, torch::Tensor slots,
+               torch::Tensor cache, int64_t seg, double eps, double temp_coef,
+               int64_t temp_every) {
+  const int kind = kind_of(q, "q");
+  CHECK_F32C(q_out);
+  TORCH_CHECK(q.dim() == 2 && q.stride(1) == 1 && q_out.dim() == 2);
+  const int T = q.size(0), wq = q.size(1);
+  TORCH_CHECK(q_out.size(0) == T && q_out.size(1) == wq);
+  CHECK_I32(positions);
+  TORCH_CHECK(positions.numel() == T);
+  const bool has_k = k.dim() == 2;
+  const bool has_v = v.numel() > 0;
+  int wk = 0, wv = 0;
+  if (eps >= 0) TORCH_CHECK(seg > 0 && wq % seg == 0, "query width / segment");
+  if (has_k) {
+    TORCH_CHECK(k.is_cuda() && k.scalar_type() == q.scalar_type() &&
+                k.dim() == 2 && k.size(0) == T && k.stride(1) == 1);
+    wk = k.size(1);
+    if (eps >= 0) TORCH_CHECK(wk % seg == 0, "key width / segment");
+    if (has_v) {
+      TORCH_CHECK(v.is_cuda() && v.scalar_type() == q.scalar_type() &&
+                  v.dim() == 2 && v.size(0) == T && v.stride(1) == 1);
+      wv = v.size(1);
+    } else {
+      wv = wk;
+    }
+    TORCH_CHECK(cache.is_cuda() && cache.scalar_type() == q.scalar_type() &&
+                cache.is_contiguous() && cache.dim() == 3 &&
+                cache.size(2) == wk + wv, "cache row width");
+    CHECK_I64(slots);
+    TORCH_CHECK(slots.numel() == T);
+  }
+  launch_qkv_store(q_out.data_ptr<float>(), q.data_ptr(), q.stride(0),
+                   has_k ? k.data_ptr() : nullptr, has_k ? k.stride(0) : 0,
+                   has_v ? v.data_ptr() : nullptr, has_v ? v.stride(0) : 0,
+                   positions.data_ptr<int>(),
+                   has_k ? slots.data_ptr<int64_t>() : nullptr,
+                   has_k ? cache.data_ptr() : nullptr, wq, wk, wv, (int)seg,
+                   (float)eps, (float)temp_coef, (int)temp_every, T, kind,
+                   cur_stream());
+}
+
+// cache [blocks, block, E]; pool [blocks, per_page, E] fp32
+void pool_cache_update(torch::Tensor cache, torch::Tensor pool,
+                       torch::Tensor block_tables, torch::Tensor token_seq,
+                       torch::Tensor positions, torch::Tensor slots, int64_t P) {
+  const int kind = kind_of(cache, "cache");
+  CHECK_F32C(pool);
+  TORCH_CHECK(cache.dim() == 3 && cache.is_contiguous() && pool.dim() == 3);
+  const int E = cache.size(2), bs = cache.size(1), per_page = pool.size(1);
+  TORCH_CHECK(P >= 1 && pool.size(2) == E && pool.size(0) == cache.size(0));
+  TORCH_CHECK((int64_t)per_page * P >= bs, "pooled rows per page");
+  CHECK_I32(block_tables);
+  CHECK_I32(positions);
+  CHECK_I64(slots);
+  const int T = positions.numel();
+  TORCH_CHECK(block_tables.dim() == 2 && slots.numel() == T);
+  const bool has_seq = token_seq.numel() > 0;
+  if (has_seq) {
+    CHECK_I32(token_seq);
+    TORCH_CHECK(token_seq.numel() == T);
+  } else {
+    TORCH_CHECK(block_tables.size(0) >= T);
+  }
+  launch_pool_cache_update(cache.data_ptr(), pool.data_ptr<float>(),
+                           block_tables.data_ptr<int>(),
+                           (int)block_tables.stride(0),
+                           has_seq ? token_seq.data_ptr<int>() : nullptr,
+                           positions.data_ptr<int>(), slots.data_ptr<int64_t>(),
+                           E, bs, per_page, (int)P, T, kind, cur_stream());
+}
+
+// out [T, H * dv] (cache type), q [T, H * M * d] fp32, cache [blocks, block,
+// G * M * d + G * dv], pool [blocks, per_page, same width] fp32 or empty
+void row_attention(torch::Tensor out, torch::Tensor q, torch::Tensor cache,
+                   torch::Tensor pool, torch::Tensor block_tables,
+                   torch::Tensor token_seq, torch::Tensor positions, int64_t H,
+                   int64_t G, int64_t M, int64_t d, int64_t dv, int64_t window,
+                   int64_t P, double scale, double softcap, double lam,
+                   double norm_eps, double out_mult, int64_t max_keys) {
+  const int kind = kind_of(cache, "cache");
+  CHECK_F32C(q);
+  TORCH_CHECK(q.dim() == 2 && cache.dim() == 3 && cache.is_contiguous());
+  const int T = q.size(0);
+  TORCH_CHECK(H >= 1 && G >= 1 && H % G == 0 && (M == 1 || M == 2) && d >= 1 &&
+              dv >= 1);
+  TORCH_CHECK(dv <= 256, "value width above 256 is not supported");
+  TORCH_CHECK(d <= 1024, "key width above 1024 is not supported");
+  TORCH_CHECK(q.size(1) == H * M * d, "query width");
+  const int E = G * M * d + G * dv;
+  TORCH_CHECK(cache.size(2) == E, "cache row width");
+  TORCH_CHECK(out.is_cuda() && out.scalar_type() == cache.scalar_type() &&
+              out.is_contiguous() && out.dim() == 2 && out.size(0) == T &&
+              out.size(1) == H * dv);
+  TORCH_CHECK(window >= 0 && P >= 0);
+  int per_page = 1;
+  const bool has_pool = window > 0 && P > 0;
+  if (has_pool) {
+    CHECK_F32C(pool);
+    TORCH_CHECK(pool.dim() == 3 && pool.size(2) == E &&
+                pool.size(0) == cache.size(0));
+    per_page = pool.size(1);
+    TORCH_CHECK((int64_t)per_page * P >= cache.size(1), "pooled rows per page");
+  }
+  CHECK_I32(block_tables);
+  CHECK_I32(positions);
+  TORCH_CHECK(block_tables.dim() == 2 && positions.numel() == T);
+  const bool has_seq = token_seq.numel() > 0;
+  if (has_seq) {
+    CHECK_I32(token_seq);
+    TORCH_CHECK(token_seq.numel() == T);
+  } else {
+    TORCH_CHECK(block_tables.size(0) >= T);
+  }
+  // shares of the key list per token: enough workgroups to fill the chip
+  // when there are few tokens (decode). Only host-known sizes enter, so a
+  // captured graph keeps its grid.
+  int64_t keys = std::max<int64_t>(1, max_keys);
+  if (window > 0) {
+    const int64_t beyond = std::max<int64_t>(0, keys - window);
+    keys = std::min<int64_t>(keys, window) + (has_pool ? beyond / P : 0);
+  }
+  const int rep = H / G;
+  const int hb = row_attention_heads_per_group(rep);
+  const int64_t wgs = (int64_t)T * G * ((rep + hb - 1) / hb);
+  int splits = 1;
+  if (wgs < 512) {
+    const int64_t by_keys = (keys + 255) / 256;  // 4 waves x 64 keys a round
+    const int64_t by_fill = (512 + wgs - 1) / std::max<int64_t>(1, wgs);
+    splits = (int)std::max<int64_t>(1, std::min<int64_t>({by_keys, by_fill, 32}));
+  }
+  torch::Tensor part;
+  if (splits > 1)
+    part = torch::empty({(int64_t)T, H, splits, M, dv + 2}, q.options());
+  launch_row_attention(
+      out.data_ptr(), splits > 1 ? part.data_ptr<float>() : nullptr,
+      q.data_ptr<float>(), cache.data_ptr(),
+      has_pool ? pool.data_ptr<float>() : nullptr, block_tables.data_ptr<int>(),
+      (int)block_tables.stride(0), has_seq ? token_seq.data_ptr<int>() : nullptr,
+      positions.data_ptr<int>(), T, (int)H, (int)G, (int)M, (int)d, (int)dv,
+      (int)cache.size(1), per_page, (int)window, has_pool ? (int)P : 0,
+      (float)scale, (float)softcap, (float)lam, (float)norm_eps,
+      (float)out_mult, splits, kind, cur_stream());
+}
+
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("add_layernorm", &add_layernorm);
   m.def("latent_kv_store", &latent_kv_store);
@@ -265,4 +504,9 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("latent_window_attention", &latent_window_attention);
   m.def("gla_recurrence", &gla_recurrence);
   m.def("gated_rmsnorm", &gated_rmsnorm);
+  m.def("sandwich_rmsnorm", &sandwich_rmsnorm);
+  m.def("xielu", &xielu);
+  m.def("qkv_store", &qkv_store);
+  m.def("pool_cache_update", &pool_cache_update);
+  m.def("row_attention", &row_attention);
 }

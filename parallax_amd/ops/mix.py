@@ -140,3 +140,105 @@ def gated_rmsnorm(o, gate, weight, eps, out_dtype):
     out = torch.empty(T, H * dv, dtype=out_dtype, device=o.device)
     _mix_ext().gated_rmsnorm(out, o, gate, weight, float(eps))
     return out
+
+
+# -- row-cache attention mixers ----------------------------------------------------
+
+
+def sandwich_rmsnorm(x, y, w_branch, hist, n_hist, dwa, w_next, eps, offset,
+                     out_dtype, add_table=None, add_index=None):
+    """One residual step of a stack that norms a branch before and after it,
+    with an optional weighted average over the outputs of all earlier layers
+    (see reference.sandwich_rmsnorm for the exact order of operations). x
+    [T, W] fp32 is updated in place; hist [n_max, T, W] fp32; dwa [n_hist]
+    fp32. Returns the normed activations in out_dtype, or None."""
+    if not x.is_cuda:
+        return ref.sandwich_rmsnorm(x, y, w_branch, hist, n_hist, dwa, w_next,
+                                    eps, offset, out_dtype, add_table, add_index)
+    ext = _mix_ext()
+    out = torch.empty(x.shape, dtype=out_dtype, device=x.device) \
+        if w_next is not None else _empty(x)
+    e = _empty(x)
+    ext.sandwich_rmsnorm(
+        x, y if y is not None else e, w_branch if y is not None else e,
+        hist if hist is not None else e, int(n_hist),
+        dwa if dwa is not None else e, w_next if w_next is not None else e,
+        float(eps), float(offset), out,
+        add_table if add_table is not None else e,
+        add_index if add_table is not None else _empty(x, torch.int32),
+    )
+    return out if w_next is not None else None
+
+
+def qkv_store(q, k, v, positions, slot_mapping, cache, seg_dim, norm_eps,
+              temp_coef, temp_every):
+    """Queries to fp32 (optionally RMS-normed per seg_dim-wide segment and
+    multiplied by a position-dependent temperature); keys (normed alike) and
+    values scattered as one row [keys | values] per token into the paged
+    cache. v None: values = the keys before the norm. k None: no store."""
+    if not q.is_cuda:
+        return ref.qkv_store(q, k, v, positions, slot_mapping, cache, seg_dim,
+                             norm_eps, temp_coef, temp_every)
+    out = torch.empty(q.shape, dtype=torch.float32, device=q.device)
+    e = _empty(q)
+    _mix_ext().qkv_store(
+        out, q, k if k is not None else e, v if v is not None else e,
+        positions, slot_mapping, cache, int(seg_dim),
+        float(norm_eps) if norm_eps is not None else -1.0,
+        float(temp_coef), int(temp_every),
+    )
+    return out
+
+
+def pool_cache_update(cache, pool, block_tables, token_seq, positions,
+                      slot_mapping, pool_tokens):
+    """Mean cache row of every block of pool_tokens positions that a token of
+    this step completes, into the fp32 pooled rows of its sequence."""
+    if not cache.is_cuda:
+        return ref.pool_cache_update(cache, pool, block_tables, token_seq,
+                                     positions, slot_mapping, pool_tokens)
+    _mix_ext().pool_cache_update(
+        cache, pool, block_tables,
+        token_seq if token_seq is not None else _empty(positions), positions,
+        slot_mapping, int(pool_tokens),
+    )
+
+
+def row_attention(q, cache, pool, block_tables, token_seq, positions, heads,
+                  kv_heads, maps, dim, vdim, window, pool_tokens, scale,
+                  softcap, lam, norm_eps, out_mult, out_dtype, max_seq_len=0):
+    """Softmax attention of fp32 queries over paged cache rows [keys |
+    values] with grouped heads: full causal (window 0) or a sliding window
+    with pooled blocks beyond it, optional tanh soft cap, one or two score
+    maps per head (two combine as a1 - lam * a2), optional RMS norm of each
+    head's result. max_seq_len: the longest context of the batch as the host
+    knows it (0 = the block tables' capacity); it only sizes the split of
+    long key ranges over workgroups. Returns [T, heads * vdim] of out_dtype."""
+    if not q.is_cuda:
+        return ref.row_attention(q, cache, pool, block_tables, token_seq,
+                                 positions, heads, kv_heads, maps, dim, vdim,
+                                 window, pool_tokens, scale, softcap, lam,
+                                 norm_eps, out_mult, out_dtype)
+    out = torch.empty(q.shape[0], heads * vdim, dtype=out_dtype, device=q.device)
+    _mix_ext().row_attention(
+        out, q, cache,
+        pool if pool is not None else torch.empty(0, dtype=torch.float32,
+                                                  device=q.device),
+        block_tables,
+        token_seq if token_seq is not None else _empty(positions), positions,
+        int(heads), int(kv_heads), int(maps), int(dim), int(vdim), int(window),
+        int(pool_tokens), float(scale), float(softcap), float(lam),
+        float(norm_eps) if norm_eps is not None else -1.0, float(out_mult),
+        int(max_seq_len) or block_tables.shape[1] * cache.shape[1],
+    )
+    return out
+
+
+def xielu(x, a_pos, a_neg):
+    """xIELU activation: a_pos z^2 + z/2 for z > 0, (1/2 + a_neg)(exp(z) - 1 -
+    z) + z/2 otherwise (fp32 inside, result in x's dtype)."""
+    if not x.is_cuda:
+        return ref.xielu(x, a_pos, a_neg)
+    out = torch.empty_like(x)
+    _mix_ext().xielu(out, x, float(a_pos), float(a_neg))
+    return out

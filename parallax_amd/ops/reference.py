@@ -655,3 +655,150 @@ def gated_rmsnorm(o, gate, weight, eps, out_dtype):
     x = o / torch.sqrt((o * o).mean(-1, keepdim=True) + eps) * weight.float()
     g = gate.float().view(T, H, dv)
     return (x * torch.nn.functional.silu(g)).view(T, H * dv).to(out_dtype)
+
+
+# -- row-cache attention mixers: sandwich RMS norm with depth averaging,
+# differential / pooled-window softmax attention over [keys | values] rows,
+# xIELU ---------------------------------------------------------------------
+
+
+def sandwich_rmsnorm(x, y, w_branch, hist, n_hist, dwa, w_next, eps, offset,
+                     out_dtype, add_table=None, add_index=None):
+    """One residual step of a stack that norms a branch before AND after it.
+    x [T, W] fp32, in place:
+      x += add_table[add_index]                       (when add_table is given)
+      x += y / rms(y) * (offset + w_branch)           (when y is given)
+      hist[n_hist - 1] = x                            (when hist is given)
+      x = sum_j dwa[j] * hist[j], j < n_hist          (when dwa is given)
+    and returns x / rms(x) * (offset + w_next) in out_dtype (None when w_next
+    is None). rms(v) = sqrt(mean(v^2) + eps); everything in fp32."""
+    if add_table is not None:
+        x.add_(add_table[add_index.long()].float())
+    if y is not None:
+        yf = y.float()
+        r = yf / torch.sqrt((yf * yf).mean(-1, keepdim=True) + eps)
+        x.add_(r * (offset + w_branch.float()))
+    if hist is not None:
+        hist[n_hist - 1].copy_(x)
+    if dwa is not None:
+        acc = torch.zeros_like(x)
+        for j in range(n_hist):
+            acc = acc + dwa[j].float() * hist[j]
+        x.copy_(acc)
+    if w_next is None:
+        return None
+    out = x / torch.sqrt((x * x).mean(-1, keepdim=True) + eps) \
+        * (offset + w_next.float())
+    return out.to(out_dtype)
+
+
+def _segment_rms(x, seg, eps):
+    T = x.shape[0]
+    v = x.view(T, -1, seg)
+    return (v / torch.sqrt((v * v).mean(-1, keepdim=True) + eps)).reshape(T, -1)
+
+
+def qkv_store(q, k, v, positions, slot_mapping, cache, seg_dim, norm_eps,
+              temp_coef, temp_every):
+    """Queries to fp32 (each seg_dim-wide segment divided by its RMS when
+    norm_eps is given; multiplied by 1 + temp_coef * ln(floor((pos + 1) /
+    temp_every) + 1) when temp_every > 0), keys (segments normed alike) and
+    values into one cache row [keys | values] per token. v None: the values
+    are the keys as they came in, before the norm. k None: nothing is stored
+    (the layer reads another layer's rows). Slot -1 skips the token."""
+    qf = q.float()
+    if norm_eps is not None:
+        qf = _segment_rms(qf, seg_dim, norm_eps)
+    if temp_every > 0:
+        p = positions.float()
+        temp = 1.0 + temp_coef * torch.log(torch.floor((p + 1.0) / temp_every) + 1.0)
+        qf = qf * temp.unsqueeze(-1)
+    if k is not None:
+        kf = k.float()
+        vals = kf if v is None else v.float()
+        if norm_eps is not None:
+            kf = _segment_rms(kf, seg_dim, norm_eps)
+        entry = torch.cat([kf, vals], dim=-1).to(cache.dtype)
+        keep = slot_mapping >= 0
+        flat = cache.view(-1, cache.shape[-1])
+        flat[slot_mapping[keep]] = entry[keep]
+    return qf.contiguous()
+
+
+def pool_cache_update(cache, pool, block_tables, token_seq, positions,
+                      slot_mapping, pool_tokens):
+    """For every token of the step that completes a block of `pool_tokens`
+    positions: the fp32 mean of the block's cache rows (as the cache holds
+    them) into the pooled rows of its sequence."""
+    T = positions.shape[0]
+    bs, per_page = cache.shape[1], pool.shape[1]
+    pos = positions.tolist()
+    seq = token_seq.tolist() if token_seq is not None else list(range(T))
+    slots = slot_mapping.tolist()
+    P = pool_tokens
+    for t in range(T):
+        p = pos[t]
+        if slots[t] < 0 or (p + 1) % P != 0:
+            continue
+        bt = block_tables[seq[t]].long()
+        j = torch.arange(p + 1 - P, p + 1)
+        rows = cache[bt[j // bs], j % bs].float()
+        acc = torch.zeros_like(rows[0])
+        for r in rows:          # in position order, as the kernel adds them
+            acc = acc + r
+        b = p // P
+        pool[bt[b // per_page], b % per_page] = acc / P
+
+
+def row_attention(q, cache, pool, block_tables, token_seq, positions, heads,
+                  kv_heads, maps, dim, vdim, window, pool_tokens, scale,
+                  softcap, lam, norm_eps, out_mult, out_dtype):
+    """Softmax attention over cache rows [keys (kv_heads x maps x dim) |
+    values (kv_heads x vdim)]. q [T, heads * maps * dim] fp32. window 0: every
+    key up to the token's position; window > 0: keys j with 0 <= pos - j <
+    window plus, when pool_tokens > 0, the pooled row of every block of
+    pool_tokens positions that ends at or before pos - window, in the same
+    softmax. softcap > 0: s <- softcap * tanh(s / softcap). maps == 2: the
+    two maps' results (same values) combine as a1 - lam * a2. norm_eps given:
+    the head's result is divided by its RMS and multiplied by out_mult.
+    Returns [T, heads * vdim] in out_dtype."""
+    T = q.shape[0]
+    bs = cache.shape[1]
+    H, G, M = heads, kv_heads, maps
+    wk = G * M * dim
+    rep = H // G
+    pos = positions.tolist()
+    seq = token_seq.tolist() if token_seq is not None else list(range(T))
+    out = torch.empty(T, H, vdim, dtype=torch.float32)
+    qv = q.view(T, G, rep, M, dim)
+    for t in range(T):
+        p = pos[t]
+        bt = block_tables[seq[t]].long()
+        lo = max(0, p - window + 1) if window > 0 else 0
+        j = torch.arange(lo, p + 1)
+        rows = cache[bt[j // bs], j % bs].float()
+        if window > 0 and pool_tokens > 0 and p - window + 1 >= pool_tokens:
+            nb = (p - window + 1) // pool_tokens
+            b = torch.arange(nb)
+            per_page = pool.shape[1]
+            rows = torch.cat([pool[bt[b // per_page], b % per_page], rows], 0)
+        k = rows[:, :wk].view(-1, G, M, dim)
+        v = rows[:, wk:].view(-1, G, vdim)
+        s = torch.einsum("grmd,ngmd->grmn", qv[t], k) * scale
+        if softcap > 0:
+            s = softcap * torch.tanh(s / softcap)
+        a = torch.einsum("grmn,ngv->grmv", torch.softmax(s, dim=-1), v)
+        o = a[:, :, 0] - lam * a[:, :, 1] if M == 2 else a[:, :, 0]
+        if norm_eps is not None:
+            o = o / torch.sqrt((o * o).mean(-1, keepdim=True) + norm_eps) * out_mult
+        out[t] = o.reshape(H, vdim)
+    return out.view(T, H * vdim).to(out_dtype)
+
+
+def xielu(x, a_pos, a_neg):
+    """z > 0: a_pos z^2 + z / 2; z <= 0: (1/2 + a_neg)(exp(z) - 1 - z) + z / 2."""
+    z = x.float()
+    neg = torch.clamp(z, max=0.0)
+    out = torch.where(z > 0, a_pos * z * z + 0.5 * z,
+                      (0.5 + a_neg) * (torch.expm1(neg) - neg) + 0.5 * z)
+    return out.to(x.dtype)

@@ -194,10 +194,12 @@ class Engine:
             latent_dims = cfg.latent_cache_dims(start, end)
             latent_ranks = [r for r, _ in latent_dims]
             latent_ropes = [d for _, d in latent_dims]
+            pool_tokens = cfg.pooled_cache_blocks(start, end)
             mla_block_bytes = max(1, MLAKVCache.bytes_per_block(
                 len(latent_dims), latent_ranks, latent_ropes,
                 args.block_size, args.dtype,
                 index_dim=cfg.index_head_dim if cfg.is_dsa else 0,
+                pool_tokens=pool_tokens,
             ))
             if args.num_kv_blocks:
                 num_blocks = args.num_kv_blocks
@@ -216,6 +218,7 @@ class Engine:
                 len(latent_dims), latent_ranks, latent_ropes,
                 args.block_size, num_blocks, self.device, mla_dtype,
                 index_dim=cfg.index_head_dim if cfg.is_dsa else 0,
+                pool_tokens=pool_tokens,
             )
         else:
             kv_dtype = args.dtype
@@ -236,7 +239,13 @@ class Engine:
             self.kv_cache = PagedKVCache(spec, num_blocks, self.device)
         self.cache_manager = CacheManager(
             args.block_size, num_blocks,
-            enable_prefix_cache=args.enable_prefix_cache and not cfg.has_linear_layers,
+            # recurrent state cannot be shared by prefix; pooled cache rows
+            # line up with their pages only when a pooled block divides a page
+            enable_prefix_cache=args.enable_prefix_cache
+            and not cfg.has_linear_layers
+            and all(p == 0 or args.block_size % p == 0
+                    for p in (cfg.pooled_cache_blocks(start, end)
+                              if self.is_mla else [])),
             num_linear_slots=(args.max_batch_size + args.extra_linear_slots)
             if cfg.has_linear_layers else 0,
         )

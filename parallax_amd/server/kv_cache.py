@@ -105,6 +105,7 @@ class MLAKVCache:
         device: torch.device,
         dtype: torch.dtype = torch.bfloat16,
         index_dim: int = 0,
+        pool_tokens=None,
     ):
         # kv_lora_rank / rope_dim may be per-layer sequences (stacks whose
         # latent layers differ in size); scalars mean every layer is alike
@@ -141,8 +142,30 @@ class MLAKVCache:
             else []
         )
 
+        # pooled rows: a layer with pool_tokens[i] = P > 0 also keeps the mean
+        # of every P consecutive rows of a sequence (fp32, whatever the cache
+        # dtype). Pooled block b of a sequence lives in the sequence's page
+        # b // per_page at offset b % per_page with per_page = ceil(block_size
+        # / P), so the ordinary block table addresses it: block b is complete
+        # only once b * P + P tokens exist, and then that page is allocated.
+        self.pool_tokens: List[int] = list(pool_tokens) if pool_tokens \
+            else [0] * num_layers
+        assert len(self.pool_tokens) == num_layers
+        self.pools: List[Optional[torch.Tensor]] = [
+            torch.zeros((num_blocks, self.pool_rows_per_block(block_size, p), r + d),
+                        dtype=torch.float32, device=device) if p > 0 else None
+            for p, r, d in zip(self.pool_tokens, ranks, ropes)
+        ]
+
+    @staticmethod
+    def pool_rows_per_block(block_size: int, pool_tokens: int) -> int:
+        return (block_size + pool_tokens - 1) // pool_tokens
+
     def layer(self, idx: int) -> torch.Tensor:
         return self.caches[idx]
+
+    def pool_layer(self, idx: int) -> Optional[torch.Tensor]:
+        return self.pools[idx]
 
     def index_layer(self, idx: int) -> torch.Tensor:
         return self.index_caches[idx]
@@ -151,10 +174,16 @@ class MLAKVCache:
     def bytes_per_block(
         num_layers: int, kv_lora_rank, rope_dim, block_size: int,
         dtype: torch.dtype = torch.bfloat16, index_dim: int = 0,
+        pool_tokens=None,
     ) -> int:
         if isinstance(kv_lora_rank, (list, tuple)):
             width = sum(kv_lora_rank) + sum(rope_dim) + index_dim * num_layers
-            return block_size * width * dtype.itemsize
+            pooled = sum(
+                MLAKVCache.pool_rows_per_block(block_size, p) * (r + d) * 4
+                for p, r, d in zip(pool_tokens or [], kv_lora_rank, rope_dim)
+                if p > 0
+            )
+            return block_size * width * dtype.itemsize + pooled
         return num_layers * block_size * (kv_lora_rank + rope_dim + index_dim) * dtype.itemsize
 
 
