@@ -206,6 +206,63 @@ def deepseek_like_config(z: dict) -> dict:
     }
 
 
+# `--design-compare --design-pair sogidra`: a Sogidra stack (pooled-window and
+# differential attention over the row cache, xIELU feed-forward, sandwich norms
+# with depth averaging) beside a Qwen3-style dense stack (grouped-query
+# attention with q/k norm, the same windows on the same layers, gated
+# feed-forward) of EQUAL sizes.
+
+SOGIDRA_SIZES = {
+    "s": dict(width=1024, layers=8, heads=16, kv_heads=4, dim=64, ff=4096,
+              window=512, pool=32, vocab=32000),
+    "m": dict(width=2048, layers=8, heads=16, kv_heads=4, dim=128, ff=8192,
+              window=1024, pool=64, vocab=32000),
+}
+
+
+def _sogidra_full_layers(z: dict):
+    """Every fourth layer (1, 5, ...) attends over the whole context."""
+    return [i for i in range(z["layers"]) if i % 4 == 1]
+
+
+def sogidra_config(z: dict) -> dict:
+    mlp = {"kind": "dense", "ff": z["ff"]}
+    full = _sogidra_full_layers(z)
+    layers = []
+    for i in range(z["layers"]):
+        if i in full:
+            # half the heads, two score maps each, values twice as wide
+            mx = {"heads": z["heads"] // 2, "kv_heads": max(1, z["kv_heads"] // 2),
+                  "dim": z["dim"], "vdim": 2 * z["dim"], "scale": z["dim"] ** -0.5,
+                  "diff": 0.3, "q_temp": {"coef": 0.1, "every": 256}}
+            if i != full[0] and full.index(i) % 2 == 1:
+                mx["kv_from"] = full[full.index(i) - 1]
+            layers.append({"type": "attention", "mixer": mx, "mlp": mlp})
+        else:
+            mx = {"heads": z["heads"], "kv_heads": z["kv_heads"], "dim": z["dim"],
+                  "vdim": z["dim"], "scale": z["dim"] ** -0.5, "softcap": 50.0,
+                  "mask": {"size": z["window"], "pool": z["pool"]}}
+            layers.append({"type": "attention_2", "mixer": mx, "mlp": mlp})
+    return {"architecture": "Sogidra", "layers": layers, "norm": {"eps": 1e-6},
+            "vocab": z["vocab"], "width": z["width"], "max_positions": 16384}
+
+
+def qwen3_like_config(z: dict) -> dict:
+    full = _sogidra_full_layers(z)
+    return {
+        "architectures": ["Qwen3ForCausalLM"], "model_type": "qwen3",
+        "vocab_size": z["vocab"], "hidden_size": z["width"],
+        "num_hidden_layers": z["layers"], "num_attention_heads": z["heads"],
+        "num_key_value_heads": z["kv_heads"], "head_dim": z["dim"],
+        "intermediate_size": z["ff"], "rms_norm_eps": 1e-6, "rope_theta": 1e6,
+        "max_position_embeddings": 16384, "tie_word_embeddings": True,
+        "sliding_window": z["window"],
+        "layer_types": ["full_attention" if i in full else "sliding_attention"
+                        for i in range(z["layers"])],
+        "torch_dtype": "bfloat16",
+    }
+
+
 def design_compare(args) -> None:
     from parallax_amd.models.config import ModelConfig
     from parallax_amd.server.engine import Engine, EngineArgs
@@ -213,9 +270,15 @@ def design_compare(args) -> None:
 
     results = []
     for size in args.design_sizes.split(","):
-        z = DESIGN_SIZES[size]
-        for design, cfg_dict in (("vurizen", vurizen_config(z)),
-                                 ("deepseek-like", deepseek_like_config(z))):
+        if args.design_pair == "sogidra":
+            z = SOGIDRA_SIZES[size]
+            pair = (("sogidra", sogidra_config(z)),
+                    ("qwen3-like", qwen3_like_config(z)))
+        else:
+            z = DESIGN_SIZES[size]
+            pair = (("vurizen", vurizen_config(z)),
+                    ("deepseek-like", deepseek_like_config(z)))
+        for design, cfg_dict in pair:
             if args.design_only and design != args.design_only:
                 continue
             cfg = ModelConfig.from_hf_config(cfg_dict)
@@ -318,12 +381,18 @@ def main():
                     help="instead of the headline workload: prefill and decode "
                          "throughput of a Vurizen stack beside a DeepSeek-V3-"
                          "style stack of equal sizes (one GPU, random weights)")
+    ap.add_argument("--design-pair", default="vurizen",
+                    choices=["vurizen", "sogidra"],
+                    help="which design --design-compare measures: vurizen "
+                         "beside a DeepSeek-V3-style stack, or sogidra beside "
+                         "a Qwen3-style dense stack")
     ap.add_argument("--design-sizes", default="s,m",
                     help="comma list of " + ",".join(DESIGN_SIZES))
     ap.add_argument("--design-batch", type=int, default=8)
     ap.add_argument("--design-prompt", type=int, default=2048)
     ap.add_argument("--design-only", default="",
-                    help="vurizen | deepseek-like (default: both)")
+                    help="one design of the pair (vurizen | deepseek-like | "
+                         "sogidra | qwen3-like; default: both)")
     args = ap.parse_args()
     if args.design_compare:
         design_compare(args)

@@ -114,6 +114,9 @@ extern "C" void launch_qkv_store(float* q_out, const void* q, int64_t q_stride,
 
 // ---- pool_cache_update -----------------------------------------------------
 
+// grid (tokens, column chunks of 256): a thread owns one column and adds the
+// block's rows in position order; the rows' offsets are looked up once per
+// workgroup (LDS) so that the loads of a column do not wait on table reads.
 template <typename T>
 __global__ __launch_bounds__(256) void pool_cache_update_kernel(
     const T* __restrict__ cache, float* __restrict__ pool,
@@ -121,6 +124,7 @@ __global__ __launch_bounds__(256) void pool_cache_update_kernel(
     const int* __restrict__ token_seq, const int* __restrict__ positions,
     const int64_t* __restrict__ slots, int E, int block_size, int per_page,
     int P) {
+  __shared__ int64_t roff[256];
   const int64_t t = blockIdx.x;
   if (slots[t] < 0) return;
   const int pos = positions[t];
@@ -128,13 +132,23 @@ __global__ __launch_bounds__(256) void pool_cache_update_kernel(
   const int b = token_seq ? token_seq[t] : (int)t;
   const int* bt = block_tables + (int64_t)b * bt_stride;
   const int blk = pos / P;
-  float* dst = pool + ((int64_t)bt[blk / per_page] * per_page + blk % per_page) * E;
-  for (int c = threadIdx.x; c < E; c += 256) {
-    float acc = 0.f;
-    for (int j = pos - P + 1; j <= pos; ++j)
-      acc += ldf(cache + ((int64_t)bt[j / block_size] * block_size + j % block_size) * E + c);
-    dst[c] = acc / (float)P;
+  const int c = blockIdx.y * 256 + threadIdx.x;
+  float acc = 0.f;
+  for (int j0 = pos - P + 1; j0 <= pos; j0 += 256) {
+    __syncthreads();
+    const int j = j0 + threadIdx.x;
+    if (j <= pos)
+      roff[threadIdx.x] = ((int64_t)bt[j / block_size] * block_size + j % block_size) * E;
+    __syncthreads();
+    const int nr = min(256, pos - j0 + 1);
+    if (c < E) {
+#pragma unroll 8
+      for (int r = 0; r < nr; ++r) acc += ldf(cache + roff[r] + c);
+    }
   }
+  if (c < E)
+    pool[((int64_t)bt[blk / per_page] * per_page + blk % per_page) * E + c] =
+        acc / (float)P;
 }
 
 extern "C" void launch_pool_cache_update(const void* cache, float* pool,
@@ -146,13 +160,13 @@ extern "C" void launch_pool_cache_update(const void* cache, float* pool,
                                          int T_, int kind, hipStream_t stream) {
   if (T_ == 0) return;
   if (kind == 0)
-    hipLaunchKernelGGL((pool_cache_update_kernel<bf16_t>), dim3(T_), dim3(256),
-                       0, stream, (const bf16_t*)cache, pool, block_tables,
+    hipLaunchKernelGGL((pool_cache_update_kernel<bf16_t>),
+                       dim3(T_, (E + 255) / 256), dim3(256), 0, stream, (const bf16_t*)cache, pool, block_tables,
                        bt_stride, token_seq, positions, slots, E, block_size,
                        per_page, P);
   else
-    hipLaunchKernelGGL((pool_cache_update_kernel<float>), dim3(T_), dim3(256), 0,
-                       stream, (const float*)cache, pool, block_tables,
+    hipLaunchKernelGGL((pool_cache_update_kernel<float>),
+                       dim3(T_, (E + 255) / 256), dim3(256), 0, stream, (const float*)cache, pool, block_tables,
                        bt_stride, token_seq, positions, slots, E, block_size,
                        per_page, P);
 }
@@ -191,7 +205,8 @@ DEVINL void ra_load4<float>(const float* p, float* v) {
   v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w;
 }
 
-// s[nq] += q[nq] . key, key = d elements at `key` (NQ queries in LDS, stride dp)
+// s[n] += q[n] . key for NQ queries in LDS that lie `dp` floats apart at
+// `qs`; key = d elements at `key`.
 template <typename TK, int NQ, bool VEC>
 DEVINL void ra_dot(const TK* __restrict__ key, const float* __restrict__ qs,
                    int dp, int d, float* s) {
@@ -336,9 +351,8 @@ __global__ __launch_bounds__(256) void row_attention_kernel(
 #pragma unroll
           for (int hh = 0; hh < HB; ++hh) sm[hh] = 0.f;
           // queries of map m sit at rows hh * M + m: stride M * dp
-          for (int hh = 0; hh < HB; ++hh)
-            ra_dot<float, 1, VEC>(pool + off + kcol + m * d,
-                                  qs + (hh * M + m) * dp, dp, d, &sm[hh]);
+          ra_dot<float, HB, VEC>(pool + off + kcol + m * d, qs + m * dp, M * dp,
+                                 d, sm);
 #pragma unroll
           for (int hh = 0; hh < HB; ++hh) s[hh * M + m] = sm[hh];
         }
@@ -350,14 +364,8 @@ __global__ __launch_bounds__(256) void row_attention_kernel(
           float sm[HB];
 #pragma unroll
           for (int hh = 0; hh < HB; ++hh) sm[hh] = 0.f;
-          if (M == 1) {
-            ra_dot<T, HB, VEC>(cache + off + kcol, qs, dp, d, sm);
-          } else {
-#pragma unroll
-            for (int hh = 0; hh < HB; ++hh)
-              ra_dot<T, 1, VEC>(cache + off + kcol + m * d,
-                                qs + (hh * M + m) * dp, dp, d, &sm[hh]);
-          }
+          ra_dot<T, HB, VEC>(cache + off + kcol + m * d, qs + m * dp, M * dp, d,
+                             sm);
 #pragma unroll
           for (int hh = 0; hh < HB; ++hh) s[hh * M + m] = sm[hh];
         }
