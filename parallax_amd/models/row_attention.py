@@ -110,6 +110,7 @@ class DifferentialAttention(_RowAttentionBase):
             meta.positions, self.heads, self.kv_heads, 2, self.dim, self.vdim,
             0, 0, self.scale, 0.0, self.lam, self.eps, 1.0 - self.diff,
             x.dtype, max_seq_len=meta.max_seq_len,
+            query_bounds=meta.query_bounds(),
         )
         return self.o_proj(o)
 
@@ -150,5 +151,6 @@ class PooledWindowAttention(_RowAttentionBase):
             meta.positions, self.heads, self.kv_heads, 1, self.dim, self.vdim,
             self.window, self.pool, self.scale, self.softcap, 0.0, None, 1.0,
             x.dtype, max_seq_len=meta.max_seq_len,
+            query_bounds=meta.query_bounds(),
         )
         return self.o_proj(o)

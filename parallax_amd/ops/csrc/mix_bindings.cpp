@@ -45,6 +45,12 @@ void launch_pool_cache_update(const void*, float*, const int*, int, const int*,
                               const int*, const int64_t*, int, int, int, int,
                               int, int, hipStream_t);
 int row_attention_heads_per_group(int);
+int row_attention_prefill_supported(int, int);
+void launch_row_attention_prefill(void*, const float*, const void*, const float*,
+                                  const int*, int, const int*, int, const int*,
+                                  int, int, int, int, int, int, int, int, int,
+                                  int, float, float, float, float, float, int,
+                                  hipStream_t);
 void launch_row_attention(void*, float*, const float*, const void*,
                           const float*, const int*, int, const int*, const int*,
                           int, int, int, int, int, int, int, int, int, int,
@@ -431,7 +437,8 @@ void row_attention(torch::Tensor out, torch::Tensor q, torch::Tensor cache,
                    torch::Tensor token_seq, torch::Tensor positions, int64_t H,
                    int64_t G, int64_t M, int64_t d, int64_t dv, int64_t window,
                    int64_t P, double scale, double softcap, double lam,
-                   double norm_eps, double out_mult, int64_t max_keys) {
+                   double norm_eps, double out_mult, int64_t max_keys,
+                   torch::Tensor query_bounds) {
   const int kind = kind_of(cache, "cache");
   CHECK_F32C(q);
   TORCH_CHECK(q.dim() == 2 && cache.dim() == 3 && cache.is_contiguous());
@@ -465,6 +472,24 @@ void row_attention(torch::Tensor out, torch::Tensor q, torch::Tensor cache,
     TORCH_CHECK(token_seq.numel() == T);
   } else {
     TORCH_CHECK(block_tables.size(0) >= T);
+  }
+  // prompt portions (token bounds per sequence given, tokens of a sequence
+  // consecutive): the matrix-core kernel, 32 tokens per workgroup
+  if (query_bounds.numel() > 0 && has_seq &&
+      row_attention_prefill_supported((int)d, (int)dv)) {
+    CHECK_I32(query_bounds);
+    const int B = query_bounds.numel() - 1;
+    TORCH_CHECK(B >= 1 && block_tables.size(0) >= B);
+    launch_row_attention_prefill(
+        out.data_ptr(), q.data_ptr<float>(), cache.data_ptr(),
+        has_pool ? pool.data_ptr<float>() : nullptr,
+        block_tables.data_ptr<int>(), (int)block_tables.stride(0),
+        query_bounds.data_ptr<int>(), B, positions.data_ptr<int>(),
+        (T + 31) / 32 + B, (int)H, (int)G, (int)M, (int)d, (int)dv,
+        (int)cache.size(1), per_page, (int)window, has_pool ? (int)P : 0,
+        (float)scale, (float)softcap, (float)lam, (float)norm_eps,
+        (float)out_mult, kind, cur_stream());
+    return;
   }
   // shares of the key list per token: enough workgroups to fill the chip
   // when there are few tokens (decode). Only host-known sizes enter, so a

@@ -1,0 +1,367 @@
+// Prompt-portion path of the row-cache attention on the fp32 matrix cores.
+//
+// Same arithmetic as row_attention.hip (fp32 scores, soft cap, softmax and
+// value sums over paged [keys | values] rows, pooled blocks beyond a sliding
+// window, one or two score maps per head), tiled for portions of many tokens:
+// a workgroup takes 32 consecutive tokens of ONE sequence, one kv head and 4
+// (head, map) streams of it, one per wave. Per step 32 keys (pooled rows
+// first, then tokens) are gathered through the block table, converted to fp32
+// and staged in LDS once for the 4 waves. Each wave then computes
+//
+//     S^T (32 keys x 32 queries) = K_tile (32 x D) . Q^T (D x 32)
+//
+// with v_mfma_f32_32x32x2_f32 (its 32 queries' features stay in registers for
+// the whole kernel). In the accumulator layout a lane holds 16 keys of ONE
+// query (column lane % 32; rows 8 i + 4 (lane / 32) + j), so mask, soft cap,
+// running max and sum are in-lane work plus one exchange with lane ^ 32, and
+// the softmax weights are already laid out as the B operand of
+//
+//     O^T (DV x 32 queries) += V_tile^T (DV x 32 keys) . P^T (32 keys x 32 queries)
+//
+// when step (i, j) of that product contracts over the key pair {8 i + j,
+// 8 i + 4 + j}: no data moves between the two products. The contraction order
+// of the first product is permuted likewise (lane half h walks features
+// h D/2 ...) so that a lane reads its key features from LDS in 16-byte pieces.
+// Key and value widths are padded with zeros to D and DV (template sizes).
+//
+// The epilogue (a1 - lam a2 for two maps, exchanged through LDS; optional RMS
+// norm over the value width; division by the softmax sum) works on columns,
+// i.e. per lane pair, too.
+#include "seq_common.h"
+
+typedef float f32x16v __attribute__((ext_vector_type(16)));
+
+#define RM_Q 32     // queries per workgroup
+#define RM_K 32     // keys per step
+#define RM_PAD 4    // LDS row padding (floats)
+
+template <typename T>
+DEVINL void rm_load8(const T* p, float* v);
+template <>
+DEVINL void rm_load8<bf16_t>(const bf16_t* p, float* v) {
+  const bf16x8 raw = load_bf16x8(p);
+#pragma unroll
+  for (int i = 0; i < 8; ++i) v[i] = bf16x8_get(raw, i);
+}
+template <>
+DEVINL void rm_load8<float>(const float* p, float* v) {
+  const float4 a = *reinterpret_cast<const float4*>(p);
+  const float4 b = *reinterpret_cast<const float4*>(p + 4);
+  v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w;
+  v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+}
+
+// D: padded key width (64 | 128), DVB: 32-wide blocks of the padded value width
+template <typename T, int M, int D, int DVB>
+__global__ __launch_bounds__(256) void row_attention_prefill_kernel(
+    T* __restrict__ out, const float* __restrict__ q, const T* __restrict__ cache,
+    const float* __restrict__ pool, const int* __restrict__ block_tables,
+    int bt_stride, const int* __restrict__ cu, int B,
+    const int* __restrict__ positions, int H, int G, int d, int dv,
+    int block_size, int per_page, int window, int P, float scale, float softcap,
+    float lam, float norm_eps, float out_mult) {
+  constexpr int DV = DVB * 32;
+  constexpr int KS = D + RM_PAD, VS = DV + RM_PAD;
+  constexpr int HW = 4 / M;  // heads per workgroup
+  extern __shared__ float lds[];
+  float* Ks = lds;                    // [M][32][KS]
+  float* Vs = lds + M * RM_K * KS;    // [32][VS]
+
+  // ---- which 32 tokens: tiles never straddle two sequences ---------------------
+  int tile = blockIdx.x, b = 0;
+  for (; b < B; ++b) {
+    const int nt = (cu[b + 1] - cu[b] + RM_Q - 1) / RM_Q;
+    if (tile < nt) break;
+    tile -= nt;
+  }
+  if (b == B) return;
+  const int t0 = cu[b] + tile * RM_Q;
+  const int nq = min(RM_Q, cu[b + 1] - t0);
+  const int p0 = positions[t0], p_last = p0 + nq - 1;
+  const int* bt = block_tables + (int64_t)b * bt_stride;
+
+  const int rep = H / G;
+  const int nhw = (rep + HW - 1) / HW;
+  const int g = blockIdx.y / nhw;
+  const int r0 = (blockIdx.y % nhw) * HW;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int half = lane >> 5, col = lane & 31;
+  const int hh = wave / M, m = wave % M;   // this wave's stream
+  const bool stream_on = r0 + hh < rep;
+  const int h = g * rep + min(r0 + hh, rep - 1);
+  const int wkeys = G * M * d;
+  const int E = wkeys + G * dv;
+  const int kcol = g * M * d, vcol = wkeys + g * dv;
+
+  // key list of the tile: pooled blocks [0, nb) then tokens [lo, p_last]
+  const int lo = window > 0 ? max(0, p0 - window + 1) : 0;
+  const int nb = (window > 0 && P > 0 && p_last - window + 1 >= P) ? (p_last - window + 1) / P : 0;
+  const int nk = nb + (p_last - lo + 1);
+
+  // the lane's query (column col): features half * D/2 + s, s < D/2
+  float qr[D / 2];
+  {
+    const bool on = stream_on && col < nq;
+    const float* src = q + (((int64_t)(t0 + min(col, nq - 1)) * H + h) * M + m) * d;
+#pragma unroll
+    for (int s = 0; s < D / 2; ++s) {
+      const int f = half * (D / 2) + s;
+      qr[s] = (on && f < d) ? src[f] : 0.f;
+    }
+  }
+  const int pq = p0 + col;
+  const bool qvalid = col < nq;
+
+  f32x16v acc[DVB];
+#pragma unroll
+  for (int k = 0; k < DVB; ++k)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[k][i] = 0.f;
+  float mx = -INFINITY, l = 0.f;
+
+  // staging role: 8 threads per key row, 8 features each per round
+  const int srow = threadIdx.x >> 3, ssub = threadIdx.x & 7;
+
+  for (int u0 = 0; u0 < nk; u0 += RM_K) {
+    __syncthreads();  // the previous step's reads are done
+    {
+      const int u = u0 + srow;
+      const bool on = u < nk;
+      const bool pooled = on && u < nb;
+      int64_t off = 0;
+      if (pooled) {
+        off = ((int64_t)bt[u / per_page] * per_page + u % per_page) * E;
+      } else if (on) {
+        const int j = lo + (u - nb);
+        off = ((int64_t)bt[j / block_size] * block_size + j % block_size) * E;
+      }
+#pragma unroll
+      for (int mm = 0; mm < M; ++mm)
+#pragma unroll
+        for (int c = 0; c < D / 64; ++c) {
+          const int f = ssub * 8 + 64 * c;
+          float v[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+          if (on && f < d) {
+            if (pooled) rm_load8<float>(pool + off + kcol + mm * d + f, v);
+            else rm_load8<T>(cache + off + kcol + mm * d + f, v);
+          }
+          float* dst = Ks + (mm * RM_K + srow) * KS + f;
+          *reinterpret_cast<float4*>(dst) = make_float4(v[0], v[1], v[2], v[3]);
+          *reinterpret_cast<float4*>(dst + 4) = make_float4(v[4], v[5], v[6], v[7]);
+        }
+#pragma unroll
+      for (int c = 0; c < (DV + 63) / 64; ++c) {
+        const int f = ssub * 8 + 64 * c;
+        if (f < DV) {
+          float v[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+          if (on && f < dv) {
+            if (pooled) rm_load8<float>(pool + off + vcol + f, v);
+            else rm_load8<T>(cache + off + vcol + f, v);
+          }
+          float* dst = Vs + srow * VS + f;
+          *reinterpret_cast<float4*>(dst) = make_float4(v[0], v[1], v[2], v[3]);
+          *reinterpret_cast<float4*>(dst + 4) = make_float4(v[4], v[5], v[6], v[7]);
+        }
+      }
+    }
+    __syncthreads();
+
+    // ---- S^T = K_tile . Q^T ---------------------------------------------------
+    f32x16v S;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) S[i] = 0.f;
+    {
+      const float* krow = Ks + (m * RM_K + col) * KS + half * (D / 2);
+#pragma unroll
+      for (int s = 0; s < D / 2; s += 4) {
+        const float4 k4 = *reinterpret_cast<const float4*>(krow + s);
+        S = __builtin_amdgcn_mfma_f32_32x32x2f32(k4.x, qr[s], S, 0, 0, 0);
+        S = __builtin_amdgcn_mfma_f32_32x32x2f32(k4.y, qr[s + 1], S, 0, 0, 0);
+        S = __builtin_amdgcn_mfma_f32_32x32x2f32(k4.z, qr[s + 2], S, 0, 0, 0);
+        S = __builtin_amdgcn_mfma_f32_32x32x2f32(k4.w, qr[s + 3], S, 0, 0, 0);
+      }
+    }
+    // ---- mask, soft cap, online softmax (column = query, 16 keys in-lane) -------
+    float tmax = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int u = u0 + 8 * i + 4 * half + j;
+        bool vis;
+        if (u < nb) {
+          vis = u * P + P - 1 <= pq - window;
+        } else {
+          const int jt = lo + (u - nb);
+          vis = jt <= pq && (window == 0 || pq - jt < window);
+        }
+        float sc = S[4 * i + j] * scale;
+        if (softcap > 0.f) sc = softcap * tanhf(sc / softcap);
+        sc = (vis && qvalid && u < nk) ? sc : -INFINITY;
+        S[4 * i + j] = sc;
+        tmax = fmaxf(tmax, sc);
+      }
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+    const float m_new = fmaxf(mx, tmax);
+    float corr = 1.f, psum = 0.f;
+    if (m_new == -INFINITY) {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) S[i] = 0.f;
+    } else {
+      corr = expf(mx - m_new);  // exp(-inf) = 0 the first time a key is seen
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const float p = expf(S[i] - m_new);  // exp(-inf) = 0 for masked keys
+        S[i] = p;
+        psum += p;
+      }
+    }
+    psum += __shfl_xor(psum, 32, 64);
+    l = l * corr + psum;
+    mx = m_new;
+    // ---- O^T += V_tile^T . P^T ------------------------------------------------
+#pragma unroll
+    for (int k = 0; k < DVB; ++k) {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) acc[k][i] *= corr;
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const float a = Vs[(8 * i + 4 * half + j) * VS + 32 * k + col];
+          acc[k] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, S[4 * i + j], acc[k], 0, 0, 0);
+        }
+    }
+  }
+
+  // ---- epilogue: lane holds O[query col][feature 32 k + 8 i + 4 half + j] --------
+  __syncthreads();  // staging area free
+  const float inv = (qvalid && l > 0.f) ? 1.0f / l : 0.f;
+  if (M == 2) {
+    // the second map's wave parks a2 (times lam) in LDS for its head's first wave
+    float* X = lds + hh * (DV * (RM_Q + 1));
+    if (m == 1) {
+#pragma unroll
+      for (int k = 0; k < DVB; ++k)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          const int f = 32 * k + 8 * (i >> 2) + 4 * half + (i & 3);
+          X[f * (RM_Q + 1) + col] = acc[k][i] * inv * lam;
+        }
+    }
+    __syncthreads();
+    if (m == 1) return;
+#pragma unroll
+    for (int k = 0; k < DVB; ++k)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const int f = 32 * k + 8 * (i >> 2) + 4 * half + (i & 3);
+        acc[k][i] = acc[k][i] * inv - X[f * (RM_Q + 1) + col];
+      }
+  } else {
+#pragma unroll
+    for (int k = 0; k < DVB; ++k)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) acc[k][i] *= inv;
+  }
+  float r = 1.0f;
+  if (norm_eps >= 0.f) {
+    float ss = 0.f;
+#pragma unroll
+    for (int k = 0; k < DVB; ++k)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) ss += acc[k][i] * acc[k][i];
+    ss += __shfl_xor(ss, 32, 64);
+    r = out_mult / sqrtf(ss / (float)dv + norm_eps);
+  }
+  if (!stream_on || !qvalid) return;
+  T* dst = out + ((int64_t)(t0 + col) * H + h) * dv;
+#pragma unroll
+  for (int k = 0; k < DVB; ++k)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int f = 32 * k + 8 * (i >> 2) + 4 * half + (i & 3);
+      if (f < dv) stf(dst + f, acc[k][i] * r);
+    }
+}
+
+struct RmArgs {
+  void* out;
+  const float* q;
+  const void* cache;
+  const float* pool;
+  const int* block_tables;
+  int bt_stride;
+  const int* cu;
+  int B;
+  const int* positions;
+  int tiles, H, G, d, dv, block_size, per_page, window, P;
+  float scale, softcap, lam, norm_eps, out_mult;
+  hipStream_t stream;
+};
+
+template <typename T, int M, int D, int DVB>
+static void launch_rm(const RmArgs& a) {
+  constexpr int DV = DVB * 32;
+  const int rep = a.H / a.G;
+  const int hw = 4 / M;
+  const size_t stage = (size_t)M * RM_K * (D + RM_PAD) + RM_K * (DV + RM_PAD);
+  const size_t xchg = M == 2 ? (size_t)hw * DV * (RM_Q + 1) : 0;
+  const size_t shm = sizeof(float) * (stage > xchg ? stage : xchg);
+  const dim3 grid(a.tiles, a.G * ((rep + hw - 1) / hw));
+  if (shm > 64 * 1024) {
+    // gfx950 has 160 KB of LDS per CU; more than 64 KB per workgroup is opt-in
+    static bool raised = false;
+    if (!raised) {
+      (void)hipFuncSetAttribute(
+          reinterpret_cast<const void*>(&row_attention_prefill_kernel<T, M, D, DVB>),
+          hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);
+      raised = true;
+    }
+  }
+  hipLaunchKernelGGL((row_attention_prefill_kernel<T, M, D, DVB>), grid,
+                     dim3(256), shm, a.stream, (T*)a.out, a.q,
+                     (const T*)a.cache, a.pool, a.block_tables, a.bt_stride,
+                     a.cu, a.B, a.positions, a.H, a.G, a.d, a.dv, a.block_size,
+                     a.per_page, a.window, a.P, a.scale, a.softcap, a.lam,
+                     a.norm_eps, a.out_mult);
+}
+
+template <typename T, int M, int D>
+static void launch_rm_d(const RmArgs& a) {
+  if (a.dv <= 64) launch_rm<T, M, D, 2>(a);
+  else if (a.dv <= 128) launch_rm<T, M, D, 4>(a);
+  else launch_rm<T, M, D, 8>(a);
+}
+
+template <typename T, int M>
+static void launch_rm_m(const RmArgs& a) {
+  if (a.d <= 64) launch_rm_d<T, M, 64>(a);
+  else launch_rm_d<T, M, 128>(a);
+}
+
+// what the matrix-core path takes: 16-byte aligned columns, widths within the
+// template sizes
+extern "C" int row_attention_prefill_supported(int d, int dv) {
+  return d % 8 == 0 && dv % 8 == 0 && d <= 128 && dv <= 256;
+}
+
+// tiles: an upper bound on the number of 32-token tiles (ceil(T / 32) + B)
+extern "C" void launch_row_attention_prefill(
+    void* out, const float* q, const void* cache, const float* pool,
+    const int* block_tables, int bt_stride, const int* cu, int B,
+    const int* positions, int tiles, int H, int G, int M, int d, int dv,
+    int block_size, int per_page, int window, int P, float scale, float softcap,
+    float lam, float norm_eps, float out_mult, int kind, hipStream_t stream) {
+  if (tiles == 0) return;
+  const RmArgs a{out, q, cache, pool, block_tables, bt_stride, cu, B, positions,
+                 tiles, H, G, d, dv, block_size, per_page, window, P, scale,
+                 softcap, lam, norm_eps, out_mult, stream};
+  if (kind == 0) {
+    if (M == 1) launch_rm_m<bf16_t, 1>(a);
+    else launch_rm_m<bf16_t, 2>(a);
+  } else {
+    if (M == 1) launch_rm_m<float, 1>(a);
+    else launch_rm_m<float, 2>(a);
+  }
+}

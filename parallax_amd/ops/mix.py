@@ -206,14 +206,18 @@ def pool_cache_update(cache, pool, block_tables, token_seq, positions,
 
 def row_attention(q, cache, pool, block_tables, token_seq, positions, heads,
                   kv_heads, maps, dim, vdim, window, pool_tokens, scale,
-                  softcap, lam, norm_eps, out_mult, out_dtype, max_seq_len=0):
+                  softcap, lam, norm_eps, out_mult, out_dtype, max_seq_len=0,
+                  query_bounds=None):
     """Softmax attention of fp32 queries over paged cache rows [keys |
     values] with grouped heads: full causal (window 0) or a sliding window
     with pooled blocks beyond it, optional tanh soft cap, one or two score
     maps per head (two combine as a1 - lam * a2), optional RMS norm of each
     head's result. max_seq_len: the longest context of the batch as the host
     knows it (0 = the block tables' capacity); it only sizes the split of
-    long key ranges over workgroups. Returns [T, heads * vdim] of out_dtype."""
+    long key ranges over workgroups. query_bounds [B+1] int32 (prompt portions:
+    tokens of sequence b are query_bounds[b] .. query_bounds[b+1], at
+    consecutive positions) lets the GPU path tile 32 tokens per workgroup on
+    the fp32 matrix cores. Returns [T, heads * vdim] of out_dtype."""
     if not q.is_cuda:
         return ref.row_attention(q, cache, pool, block_tables, token_seq,
                                  positions, heads, kv_heads, maps, dim, vdim,
@@ -230,6 +234,8 @@ def row_attention(q, cache, pool, block_tables, token_seq, positions, heads,
         int(pool_tokens), float(scale), float(softcap), float(lam),
         float(norm_eps) if norm_eps is not None else -1.0, float(out_mult),
         int(max_seq_len) or block_tables.shape[1] * cache.shape[1],
+        query_bounds if query_bounds is not None and token_seq is not None
+        else _empty(positions),
     )
     return out
 

@@ -52,6 +52,7 @@ mix_sources = [
     os.path.join(CSRC, "gla.hip"),
     os.path.join(CSRC, "sandwich_norm.hip"),
     os.path.join(CSRC, "row_attention.hip"),
+    os.path.join(CSRC, "row_attention_mfma.hip"),
 ]
 
 wanted = [x for x in os.environ.get("PARALLAX_EXT", "_C,_mix").split(",") if x]

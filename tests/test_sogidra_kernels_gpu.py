@@ -173,6 +173,9 @@ CASES = [
     (2, 2, 2, 12, 10, 0, 0, 0.0, True),        # scalar path
     (4, 1, 2, 64, 128, 0, 0, 0.0, True),
     (2, 1, 1, 8, 256, 50, 0, 0.0, False),      # window without pooled blocks
+    (2, 1, 2, 128, 256, 0, 0, 0.0, True),      # the widest the matrix-core path takes
+    (5, 1, 1, 48, 96, 40, 8, 20.0, False),     # widths padded to the tile sizes
+    (4, 4, 1, 136, 64, 0, 0, 0.0, False),      # keys wider than the matrix-core path
 ]
 
 
@@ -192,12 +195,14 @@ def test_row_attention(dtype, case, decode):
             pos, seq, slots = _step(pg, [(s, 0, n)])
             ref.pool_cache_update(pg.cache, pg.pool, pg.block_tables, seq, pos,
                                   slots, P)
+    bounds = None
     if decode:
         pos = torch.tensor([n - 1 for n in lens], dtype=torch.int32)
         seq = None
         max_len = max(lens)
     else:
         pos, seq, _ = _step(pg, [(0, 250, 50), (1, 0, 77), (2, 0, 1)])
+        bounds = torch.tensor([0, 50, 127, 128], dtype=torch.int32)
         max_len = max(lens)
     T = pos.numel()
     q = _rand(T, H * M * d, seed=8)
@@ -209,8 +214,15 @@ def test_row_attention(dtype, case, decode):
     dd = lambda t: t.to(DEV) if t is not None else None
     got = ops.row_attention(dd(q), dd(pg.cache), dd(pg.pool),
                             dd(pg.block_tables), dd(seq), dd(pos), *args, dtype,
-                            max_seq_len=max_len)
+                            max_seq_len=max_len, query_bounds=dd(bounds))
     assert got.dtype == dtype
+    if not decode:
+        # the same tokens without their bounds: one workgroup per token
+        per_token = ops.row_attention(dd(q), dd(pg.cache), dd(pg.pool),
+                                      dd(pg.block_tables), dd(seq), dd(pos),
+                                      *args, dtype, max_seq_len=max_len)
+        rt, at = _tol(dtype)
+        torch.testing.assert_close(per_token.float().cpu(), want, rtol=rt, atol=at)
     rt, at = _tol(dtype)
     torch.testing.assert_close(got.float().cpu(), want, rtol=rt, atol=at)
     if decode:
