@@ -51,6 +51,42 @@ DEVINL void rm_load8<float>(const float* p, float* v) {
   v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
 }
 
+// 8 cache elements as they are loaded (converted only when they go to LDS, so
+// that a prefetched tile costs few registers while the loads are in flight)
+template <typename T>
+struct rm_raw8;
+template <>
+struct rm_raw8<bf16_t> {
+  int4 v;
+  DEVINL void fetch(const bf16_t* p) { v = *reinterpret_cast<const int4*>(p); }
+  DEVINL void zero() { v = make_int4(0, 0, 0, 0); }
+  DEVINL void unpack(float* o) const {
+    bf16x8 r;
+    r.raw = v;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) o[i] = bf16x8_get(r, i);
+  }
+};
+template <>
+struct rm_raw8<float> {
+  float4 a, b;
+  DEVINL void fetch(const float* p) {
+    a = *reinterpret_cast<const float4*>(p);
+    b = *reinterpret_cast<const float4*>(p + 4);
+  }
+  DEVINL void zero() { a = b = make_float4(0.f, 0.f, 0.f, 0.f); }
+  DEVINL void unpack(float* o) const {
+    o[0] = a.x; o[1] = a.y; o[2] = a.z; o[3] = a.w;
+    o[4] = b.x; o[5] = b.y; o[6] = b.z; o[7] = b.w;
+  }
+};
+
+// tanh through one exponential and one reciprocal (both hardware
+// approximations, relative error about 1e-6; +-1 at the ends)
+DEVINL float rm_tanh(float x) {
+  return 1.0f - 2.0f * __frcp_rn(__expf(2.0f * x) + 1.0f);
+}
+
 // D: padded key width (64 | 128), DVB: 32-wide blocks of the padded value width
 template <typename T, int M, int D, int DVB>
 __global__ __launch_bounds__(256) void row_attention_prefill_kernel(
@@ -118,13 +154,70 @@ __global__ __launch_bounds__(256) void row_attention_prefill_kernel(
 #pragma unroll
     for (int i = 0; i < 16; ++i) acc[k][i] = 0.f;
   float mx = -INFINITY, l = 0.f;
+  const float inv_cap = softcap > 0.f ? 1.0f / softcap : 0.f;
 
   // staging role: 8 threads per key row, 8 features each per round
   const int srow = threadIdx.x >> 3, ssub = threadIdx.x & 7;
 
+  // steps whose 32 keys are all token rows (every step after the pooled rows)
+  // are prefetched: their global loads are issued before the previous step's
+  // products and land in LDS after them
+  constexpr int KC = D / 64, VC = (DV + 63) / 64;
+  rm_raw8<T> kraw[M][KC], vraw[VC];
+  auto fetch = [&](int u0) {
+    const int u = u0 + srow;
+    const bool on = u < nk;
+    int64_t off = 0;
+    if (on) {
+      const int j = lo + (u - nb);
+      off = ((int64_t)bt[j / block_size] * block_size + j % block_size) * E;
+    }
+#pragma unroll
+    for (int mm = 0; mm < M; ++mm)
+#pragma unroll
+      for (int c = 0; c < KC; ++c) {
+        const int f = ssub * 8 + 64 * c;
+        if (on && f < d) kraw[mm][c].fetch(cache + off + kcol + mm * d + f);
+        else kraw[mm][c].zero();
+      }
+#pragma unroll
+    for (int c = 0; c < VC; ++c) {
+      const int f = ssub * 8 + 64 * c;
+      if (on && f < dv) vraw[c].fetch(cache + off + vcol + f);
+      else vraw[c].zero();
+    }
+  };
+  auto stash = [&]() {
+#pragma unroll
+    for (int mm = 0; mm < M; ++mm)
+#pragma unroll
+      for (int c = 0; c < KC; ++c) {
+        float v[8];
+        kraw[mm][c].unpack(v);
+        float* dst = Ks + (mm * RM_K + srow) * KS + ssub * 8 + 64 * c;
+        *reinterpret_cast<float4*>(dst) = make_float4(v[0], v[1], v[2], v[3]);
+        *reinterpret_cast<float4*>(dst + 4) = make_float4(v[4], v[5], v[6], v[7]);
+      }
+#pragma unroll
+    for (int c = 0; c < VC; ++c) {
+      const int f = ssub * 8 + 64 * c;
+      if (f < DV) {
+        float v[8];
+        vraw[c].unpack(v);
+        float* dst = Vs + srow * VS + f;
+        *reinterpret_cast<float4*>(dst) = make_float4(v[0], v[1], v[2], v[3]);
+        *reinterpret_cast<float4*>(dst + 4) = make_float4(v[4], v[5], v[6], v[7]);
+      }
+    }
+  };
+
+  bool fetched = false;
   for (int u0 = 0; u0 < nk; u0 += RM_K) {
     __syncthreads();  // the previous step's reads are done
-    {
+    if (u0 >= nb) {
+      if (!fetched) fetch(u0);
+      stash();
+    } else {
       const int u = u0 + srow;
       const bool on = u < nk;
       const bool pooled = on && u < nb;
@@ -165,6 +258,8 @@ __global__ __launch_bounds__(256) void row_attention_prefill_kernel(
       }
     }
     __syncthreads();
+    fetched = u0 + RM_K < nk && u0 + RM_K >= nb;
+    if (fetched) fetch(u0 + RM_K);
 
     // ---- S^T = K_tile . Q^T ---------------------------------------------------
     f32x16v S;
@@ -182,25 +277,40 @@ __global__ __launch_bounds__(256) void row_attention_prefill_kernel(
       }
     }
     // ---- mask, soft cap, online softmax (column = query, 16 keys in-lane) -------
+    // a step whose 32 keys are tokens that every one of the 32 queries sees
+    // needs no mask (most steps of a long portion)
+    const int jt0 = lo + (u0 - nb);
+    const bool interior = nq == RM_Q && u0 >= nb && u0 + RM_K <= nk &&
+                          jt0 + RM_K - 1 <= p0 && (window == 0 || p_last - jt0 < window);
     float tmax = -INFINITY;
+    if (interior) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const int u = u0 + 8 * i + 4 * half + j;
-        bool vis;
-        if (u < nb) {
-          vis = u * P + P - 1 <= pq - window;
-        } else {
-          const int jt = lo + (u - nb);
-          vis = jt <= pq && (window == 0 || pq - jt < window);
-        }
-        float sc = S[4 * i + j] * scale;
-        if (softcap > 0.f) sc = softcap * tanhf(sc / softcap);
-        sc = (vis && qvalid && u < nk) ? sc : -INFINITY;
-        S[4 * i + j] = sc;
+      for (int i = 0; i < 16; ++i) {
+        float sc = S[i] * scale;
+        if (softcap > 0.f) sc = softcap * rm_tanh(sc * inv_cap);
+        S[i] = sc;
         tmax = fmaxf(tmax, sc);
       }
+    } else {
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const int u = u0 + 8 * i + 4 * half + j;
+          bool vis;
+          if (u < nb) {
+            vis = u * P + P - 1 <= pq - window;
+          } else {
+            const int jt = lo + (u - nb);
+            vis = jt <= pq && (window == 0 || pq - jt < window);
+          }
+          float sc = S[4 * i + j] * scale;
+          if (softcap > 0.f) sc = softcap * rm_tanh(sc * inv_cap);
+          sc = (vis && qvalid && u < nk) ? sc : -INFINITY;
+          S[4 * i + j] = sc;
+          tmax = fmaxf(tmax, sc);
+        }
+    }
     tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
     const float m_new = fmaxf(mx, tmax);
     float corr = 1.f, psum = 0.f;
@@ -208,10 +318,10 @@ __global__ __launch_bounds__(256) void row_attention_prefill_kernel(
 #pragma unroll
       for (int i = 0; i < 16; ++i) S[i] = 0.f;
     } else {
-      corr = expf(mx - m_new);  // exp(-inf) = 0 the first time a key is seen
+      corr = __expf(mx - m_new);  // exp(-inf) = 0 the first time a key is seen
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
-        const float p = expf(S[i] - m_new);  // exp(-inf) = 0 for masked keys
+        const float p = __expf(S[i] - m_new);  // exp(-inf) = 0 for masked keys
         S[i] = p;
         psum += p;
       }
