@@ -211,6 +211,7 @@ template <typename TK, int NQ, bool VEC>
 DEVINL void ra_dot(const TK* __restrict__ key, const float* __restrict__ qs,
                    int dp, int d, float* s) {
   if (VEC) {
+#pragma unroll 2
     for (int f = 0; f < d; f += 8) {
       float kv[8];
       ra_load8<TK>(key + f, kv);
@@ -393,6 +394,7 @@ __global__ __launch_bounds__(256) void row_attention_kernel(
 #pragma unroll
       for (int i = 0; i < 4; ++i) acc[n][i] *= corr[n];
     const int cnt = min(64, nk - u0);
+#pragma unroll 4
     for (int jj = ks; jj < cnt; jj += kp) {
       const int64_t r = rows[jj];
       float vv[4];
@@ -501,35 +503,50 @@ __global__ __launch_bounds__(256) void row_attention_kernel(
   }
 }
 
-// one wave per (token, head): joins `splits` partial results, then the epilogue
+// one wave per (token, head): joins `splits` (at most 64) partial results, then
+// the epilogue. Lane s weighs split s once; every lane then adds up its value
+// features over the splits.
 template <typename T, int M>
 __global__ __launch_bounds__(64) void row_attention_reduce_kernel(
     T* __restrict__ out, const float* __restrict__ part, int dv, int splits,
     float lam, float norm_eps, float out_mult) {
-  extern __shared__ float lds[];  // [M][dvp]
+  extern __shared__ float lds[];  // [M][dvp] sums | [M][64] weights
   const int64_t th = blockIdx.x;
   const int lane = threadIdx.x;
   const int dvp = (dv + 3) & ~3;
+  float* wts = lds + M * dvp;
+  const int64_t step = (int64_t)M * (dv + 2);
   float lg[M];
 #pragma unroll
   for (int m = 0; m < M; ++m) {
     const float* pr = part + (th * splits * M + m) * (int64_t)(dv + 2);
-    const int64_t step = (int64_t)M * (dv + 2);
-    float mg = -INFINITY;
-    for (int s = 0; s < splits; ++s) mg = fmaxf(mg, pr[s * step]);
-    float a = 0.f;
+    const float ms = lane < splits ? pr[lane * step] : -INFINITY;
+    const float ls = lane < splits ? pr[lane * step + 1] : 0.f;
+    const float mg = wave_reduce_max(ms);
+    const float w = (ms == -INFINITY) ? 0.f : expf(ms - mg);
+    lg[m] = wave_reduce_sum(ls * w);
+    wts[m * 64 + lane] = w;
+  }
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+  for (int m = 0; m < M; ++m) {
+    const float* pr = part + (th * splits * M + m) * (int64_t)(dv + 2) + 2;
+    float v[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll 4
     for (int s = 0; s < splits; ++s) {
-      const float ms = pr[s * step];
-      a += (ms == -INFINITY) ? 0.f : pr[s * step + 1] * expf(ms - mg);
-    }
-    lg[m] = a;
-    for (int f = lane; f < dv; f += 64) {
-      float v = 0.f;
-      for (int s = 0; s < splits; ++s) {
-        const float ms = pr[s * step];
-        if (ms != -INFINITY) v += pr[s * step + 2 + f] * expf(ms - mg);
+      const float w = wts[m * 64 + s];
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        const int f = lane + 64 * c;
+        if (f < dv) v[c] = fmaf(w, pr[s * step + f], v[c]);
       }
-      lds[m * dvp + f] = v;
+    }
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      const int f = lane + 64 * c;
+      if (f < dv) lds[m * dvp + f] = v[c];
     }
   }
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
@@ -581,7 +598,7 @@ static void launch_ra_hb(const RaArgs& a) {
 #undef RA_CALL
   if (a.splits > 1)
     hipLaunchKernelGGL((row_attention_reduce_kernel<T, M>),
-                       dim3(a.T_ * a.H), dim3(64), sizeof(float) * M * dvp,
+                       dim3(a.T_ * a.H), dim3(64), sizeof(float) * M * (dvp + 64),
                        a.stream, (T*)a.out, a.part, a.dv, a.splits, a.lam,
                        a.norm_eps, a.out_mult);
 }

@@ -85,6 +85,148 @@ __global__ __launch_bounds__(256) void sandwich_rmsnorm_kernel(
 #undef SN_CUR
 }
 
+// ---- rows whose width is a multiple of 4 and at most 4096: 16-byte accesses -----
+template <typename T>
+DEVINL void sn_load4(const T* p, float* v);
+template <>
+DEVINL void sn_load4<float>(const float* p, float* v) {
+  const float4 a = *reinterpret_cast<const float4*>(p);
+  v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w;
+}
+template <>
+DEVINL void sn_load4<bf16_t>(const bf16_t* p, float* v) {
+  const uint2 raw = *reinterpret_cast<const uint2*>(p);
+  v[0] = bf16_bits_to_f32((uint16_t)(raw.x & 0xffff));
+  v[1] = bf16_bits_to_f32((uint16_t)(raw.x >> 16));
+  v[2] = bf16_bits_to_f32((uint16_t)(raw.y & 0xffff));
+  v[3] = bf16_bits_to_f32((uint16_t)(raw.y >> 16));
+}
+template <typename T>
+DEVINL void sn_store4(T* p, const float* v);
+template <>
+DEVINL void sn_store4<float>(float* p, const float* v) {
+  *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
+}
+template <>
+DEVINL void sn_store4<bf16_t>(bf16_t* p, const float* v) {
+  uint2 raw;
+  raw.x = (uint32_t)f32_to_bf16_bits(v[0]) | ((uint32_t)f32_to_bf16_bits(v[1]) << 16);
+  raw.y = (uint32_t)f32_to_bf16_bits(v[2]) | ((uint32_t)f32_to_bf16_bits(v[3]) << 16);
+  *reinterpret_cast<uint2*>(p) = raw;
+}
+
+#define SN_NC 4  // 4-element pieces per thread
+
+// Same steps as above. The history loop runs over the earlier layers on the
+// outside and over the thread's pieces on the inside, so that the loads of
+// one history row are in flight together.
+template <typename TY, typename TP>
+__global__ __launch_bounds__(256) void sandwich_rmsnorm_vec4_kernel(
+    float* __restrict__ x, const TY* __restrict__ y, int64_t y_stride,
+    const TP* __restrict__ wb, float* __restrict__ hist, int64_t hist_stride,
+    int n_hist, const float* __restrict__ dwa, const TP* __restrict__ wn,
+    float eps, float offset, TP* __restrict__ out,
+    const TP* __restrict__ add_table, const int* __restrict__ add_index, int W) {
+  __shared__ float scratch[8];
+  const int64_t row = blockIdx.x;
+  float* xr = x + row * W;
+  float v[SN_NC][4];
+  bool on[SN_NC];
+  int at[SN_NC];
+#pragma unroll
+  for (int c = 0; c < SN_NC; ++c) {
+    at[c] = (threadIdx.x + 256 * c) * 4;
+    on[c] = at[c] < W;
+    if (on[c]) sn_load4<float>(xr + at[c], v[c]);
+    else v[c][0] = v[c][1] = v[c][2] = v[c][3] = 0.f;
+  }
+  if (add_table) {
+    const TP* trow = add_table + (int64_t)add_index[row] * W;
+#pragma unroll
+    for (int c = 0; c < SN_NC; ++c)
+      if (on[c]) {
+        float t[4];
+        sn_load4<TP>(trow + at[c], t);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) v[c][i] += t[i];
+      }
+  }
+  if (y) {
+    const TY* yr = y + row * y_stride;
+    float yv[SN_NC][4];
+    float ss = 0.f;
+#pragma unroll
+    for (int c = 0; c < SN_NC; ++c) {
+      if (on[c]) sn_load4<TY>(yr + at[c], yv[c]);
+      else yv[c][0] = yv[c][1] = yv[c][2] = yv[c][3] = 0.f;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) ss += yv[c][i] * yv[c][i];
+    }
+    const float rinv = 1.0f / sqrtf(block256_sum(ss, scratch) / (float)W + eps);
+#pragma unroll
+    for (int c = 0; c < SN_NC; ++c)
+      if (on[c]) {
+        float w4[4];
+        sn_load4<TP>(wb + at[c], w4);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) v[c][i] += yv[c][i] * rinv * (offset + w4[i]);
+      }
+  }
+  if (hist) {
+    float* hr = hist + (int64_t)(n_hist - 1) * hist_stride + row * W;
+#pragma unroll
+    for (int c = 0; c < SN_NC; ++c)
+      if (on[c]) sn_store4<float>(hr + at[c], v[c]);
+  }
+  if (dwa) {
+    float acc[SN_NC][4];
+#pragma unroll
+    for (int c = 0; c < SN_NC; ++c)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) acc[c][i] = 0.f;
+#pragma unroll 4
+    for (int j = 0; j < n_hist - 1; ++j) {
+      const float wj = dwa[j];
+      const float* hj = hist + (int64_t)j * hist_stride + row * W;
+#pragma unroll
+      for (int c = 0; c < SN_NC; ++c)
+        if (on[c]) {
+          float t[4];
+          sn_load4<float>(hj + at[c], t);
+#pragma unroll
+          for (int i = 0; i < 4; ++i) acc[c][i] = fmaf(wj, t[i], acc[c][i]);
+        }
+    }
+    const float wl = dwa[n_hist - 1];
+#pragma unroll
+    for (int c = 0; c < SN_NC; ++c)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) v[c][i] = fmaf(wl, v[c][i], acc[c][i]);
+  }
+  if (add_table || y || dwa) {
+#pragma unroll
+    for (int c = 0; c < SN_NC; ++c)
+      if (on[c]) sn_store4<float>(xr + at[c], v[c]);
+  }
+  if (wn == nullptr) return;
+  float ss = 0.f;
+#pragma unroll
+  for (int c = 0; c < SN_NC; ++c)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) ss += v[c][i] * v[c][i];
+  const float rinv = 1.0f / sqrtf(block256_sum(ss, scratch) / (float)W + eps);
+  TP* o = out + row * W;
+#pragma unroll
+  for (int c = 0; c < SN_NC; ++c)
+    if (on[c]) {
+      float w4[4], r[4];
+      sn_load4<TP>(wn + at[c], w4);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) r[i] = v[c][i] * rinv * (offset + w4[i]);
+      sn_store4<TP>(o + at[c], r);
+    }
+}
+
 template <typename TY, typename TP>
 static void launch_sn_t(float* x, const void* y, int64_t y_stride,
                         const void* wb, float* hist, int64_t hist_stride,
@@ -93,7 +235,14 @@ static void launch_sn_t(float* x, const void* y, int64_t y_stride,
                         const int* add_index, int rows, int W,
                         hipStream_t stream) {
   if (rows == 0) return;
-  if (W <= 256 * SN_NV)
+  if (W % 4 == 0 && W <= 256 * 4 * SN_NC && y_stride % 4 == 0 &&
+      reinterpret_cast<uintptr_t>(y) % 16 == 0)
+    hipLaunchKernelGGL((sandwich_rmsnorm_vec4_kernel<TY, TP>), dim3(rows),
+                       dim3(256), 0, stream, x, (const TY*)y, y_stride,
+                       (const TP*)wb, hist, hist_stride, n_hist, dwa,
+                       (const TP*)wn, eps, offset, (TP*)out,
+                       (const TP*)add_table, add_index, W);
+  else if (W <= 256 * SN_NV)
     hipLaunchKernelGGL((sandwich_rmsnorm_kernel<TY, TP, true>), dim3(rows),
                        dim3(256), 0, stream, x, (const TY*)y, y_stride,
                        (const TP*)wb, hist, hist_stride, n_hist, dwa,
