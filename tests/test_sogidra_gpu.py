@@ -114,6 +114,31 @@ def test_sizes_outside_the_tuned_gemm_path(tmp_path, dtype):
         U.describe(got, oracle.forward(cfg, w, toks), TOL[dtype])
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_widths_the_matrix_core_path_pads(tmp_path, dtype):
+    """Key and value widths that are multiples of 8 but not of the matrix-core
+    tiles (40, 24 / 72, 104), head groups of 3, 5 and 6, a pooled block longer
+    than its window, a window of one token: long portions take the tiled
+    kernel, single tokens the per-token one, and both agree with the
+    reference."""
+    layers = [U.window_spec(6, 2, 40, size=10, pool=4, softcap=5.0, mlp=U.dense(48)),
+              U.diff_spec(3, 1, 24, 72, scale=0.2, every=5, mlp=None),
+              U.window_spec(5, 1, 104, size=3, pool=7, softcap=0.0, scale=0.1),
+              U.diff_spec(6, 1, 24, 72, kv_from=1, scale=0.15, diff=0.4, mlp=U.dense(48)),
+              U.window_spec(4, 4, 8, size=1, pool=2, mlp=None)]
+    cfg = U.small_config(layers, width=56, vocab=61)
+    w = oracle.random_weights(cfg, seed=23)
+    path = U.write_checkpoint(str(tmp_path), cfg, w)
+    eng = U.make_engine(path, device="cuda", dtype=dtype, pages=40)
+    seqs = {"a": U.tokens(140, 61, 31), "b": U.tokens(45, 61, 32)}
+    schedule = [[("a", 70)], [("a", 33), ("b", 40)], [("a", 1), ("b", 1)],
+                [("a", 36), ("b", 4)]]
+    got = U.run_schedule(eng, seqs, schedule)
+    for name, toks in seqs.items():
+        want = oracle.forward(cfg, w, toks)
+        assert close(got[name], want, dtype), (name, U.describe(got[name], want, TOL[dtype]))
+
+
 def test_greedy_generation_fp32_matches_the_reference(ckpt):
     cfg, w, path = ckpt
     eng = U.make_engine(path, device="cuda", dtype=torch.float32, prefill_chunk_size=16)
