@@ -234,13 +234,13 @@ def sogidra_config(z: dict) -> dict:
             # half the heads, two score maps each, values twice as wide
             mx = {"heads": z["heads"] // 2, "kv_heads": max(1, z["kv_heads"] // 2),
                   "dim": z["dim"], "vdim": 2 * z["dim"], "scale": z["dim"] ** -0.5,
-                  "diff": 0.3, "q_temp": {"coef": 0.1, "every": 256}}
+                  "diff": 0.2, "q_temp": {"coef": 0.1, "every": 256}}
             if i != full[0] and full.index(i) % 2 == 1:
                 mx["kv_from"] = full[full.index(i) - 1]
             layers.append({"type": "attention", "mixer": mx, "mlp": mlp})
         else:
             mx = {"heads": z["heads"], "kv_heads": z["kv_heads"], "dim": z["dim"],
-                  "vdim": z["dim"], "scale": z["dim"] ** -0.5, "softcap": 50.0,
+                  "vdim": z["dim"], "scale": z["dim"] ** -0.5, "softcap": 30.0,
                   "mask": {"size": z["window"], "pool": z["pool"]}}
             layers.append({"type": "attention_2", "mixer": mx, "mlp": mlp})
     return {"architecture": "Sogidra", "layers": layers, "norm": {"eps": 1e-6},

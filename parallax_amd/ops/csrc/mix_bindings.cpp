@@ -504,7 +504,7 @@ void row_attention(torch::Tensor out, torch::Tensor q, torch::Tensor cache,
   const int64_t wgs = (int64_t)T * G * ((rep + hb - 1) / hb);
   int splits = 1;
   if (wgs < 512) {
-    const int64_t by_keys = (keys + 255) / 256;  // 4 waves x 64 keys a round
+    const int64_t by_keys = (keys + 255) / 256;  // 4 waves x 64 keys per pass
     const int64_t by_fill = (512 + wgs - 1) / std::max<int64_t>(1, wgs);
     splits = (int)std::max<int64_t>(1, std::min<int64_t>({by_keys, by_fill, 32}));
   }

@@ -156,7 +156,7 @@ __global__ __launch_bounds__(256) void row_attention_prefill_kernel(
   float mx = -INFINITY, l = 0.f;
   const float inv_cap = softcap > 0.f ? 1.0f / softcap : 0.f;
 
-  // staging role: 8 threads per key row, 8 features each per round
+  // staging role: 8 threads per key row, 8 features each at a time
   const int srow = threadIdx.x >> 3, ssub = threadIdx.x & 7;
 
   // steps whose 32 keys are all token rows (every step after the pooled rows)

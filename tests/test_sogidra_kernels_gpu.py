@@ -168,7 +168,7 @@ CASES = [
     (4, 2, 1, 32, 32, 20, 4, 30.0, False),     # pooled window, vector path
     (6, 2, 1, 24, 24, 33, 5, 0.0, False),      # block does not divide a page
     (3, 3, 1, 20, 20, 7, 1, 10.0, False),      # scalar path, blocks of one token
-    (8, 1, 1, 64, 64, 200, 16, 50.0, False),   # eight heads share one kv head
+    (8, 1, 1, 64, 64, 200, 32, 40.0, False),   # eight heads share one kv head
     (4, 2, 2, 16, 40, 0, 0, 0.0, True),        # two maps, full causal, head norm
     (2, 2, 2, 12, 10, 0, 0, 0.0, True),        # scalar path
     (4, 1, 2, 64, 128, 0, 0, 0.0, True),
