@@ -89,7 +89,7 @@ DEVINL float rm_tanh(float x) {
 
 // D: padded key width (64 | 128), DVB: 32-wide blocks of the padded value width
 template <typename T, int M, int D, int DVB>
-__global__ __launch_bounds__(256) void row_attention_prefill_kernel(
+__global__ __launch_bounds__(256, 2) void row_attention_prefill_kernel(
     T* __restrict__ out, const float* __restrict__ q, const T* __restrict__ cache,
     const float* __restrict__ pool, const int* __restrict__ block_tables,
     int bt_stride, const int* __restrict__ cu, int B,
@@ -211,6 +211,8 @@ __global__ __launch_bounds__(256) void row_attention_prefill_kernel(
     }
   };
 
+  // the widest value tile leaves no registers for a tile in flight
+  constexpr bool PREFETCH = DVB <= 4;
   bool fetched = false;
   for (int u0 = 0; u0 < nk; u0 += RM_K) {
     __syncthreads();  // the previous step's reads are done
@@ -258,7 +260,7 @@ __global__ __launch_bounds__(256) void row_attention_prefill_kernel(
       }
     }
     __syncthreads();
-    fetched = u0 + RM_K < nk && u0 + RM_K >= nb;
+    fetched = PREFETCH && u0 + RM_K < nk && u0 + RM_K >= nb;
     if (fetched) fetch(u0 + RM_K);
 
     // ---- S^T = K_tile . Q^T ---------------------------------------------------
