@@ -124,10 +124,10 @@ class ModelConfig:
                 if sp["type"] == "latent_attention":
                     dims.append((int(mx["kv_rank"]), int(mx["rot_dim"])))
                 elif sp["type"] == "attention":      # two score maps per head
-                    g = int(mx["kv_heads"])
+                    g = int(mx.get("kv_heads", mx["heads"]))
                     dims.append((g * 2 * int(mx["dim"]), g * int(mx["vdim"])))
                 elif sp["type"] == "attention_2":    # values = unnormed keys
-                    g = int(mx["kv_heads"])
+                    g = int(mx.get("kv_heads", mx["heads"]))
                     dims.append((g * int(mx["dim"]), g * int(mx["dim"])))
             return dims
         if not self.is_mla:
@@ -223,8 +223,12 @@ class ModelConfig:
         linear = [sp["mixer"] for sp in layers if sp["type"] == "gla"]
         windowed = [sp["mixer"] for sp in layers if sp["type"] == "attention_2"]
         mlps = [sp["mlp"] for sp in layers if sp.get("mlp") is not None]
-        moes = [m for m in mlps if m.get("kind", "moe") == "moe"]
-        dense = [m for m in mlps if m.get("kind", "moe") == "dense"]
+
+        def kind_of(m):   # a feed-forward without a router is a dense one
+            return m.get("kind", "moe" if "router" in m else "dense")
+
+        moes = [m for m in mlps if kind_of(m) == "moe"]
+        dense = [m for m in mlps if kind_of(m) == "dense"]
         first = layers[0]["mixer"]
         mc = cls(
             architecture=cfg["architecture"],

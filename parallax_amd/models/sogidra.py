@@ -150,17 +150,17 @@ class SogidraShardModel(nn.Module):
             if spec["type"] == "attention":
                 temp = mx.get("q_temp") or {}
                 mixer = DifferentialAttention(
-                    W, int(mx["heads"]), int(mx["kv_heads"]), int(mx["dim"]),
-                    int(mx["vdim"]), float(mx["scale"]), float(mx["diff"]),
+                    W, int(mx["heads"]), int(mx.get("kv_heads", mx["heads"])), int(mx["dim"]),
+                    int(mx["vdim"]), float(mx["scale"]), float(mx.get("diff", 0.0)),
                     float(temp.get("coef", 0.0)), int(temp.get("every", 0)),
                     eps, idx, owns,
                 )
             elif spec["type"] == "attention_2":
                 mask = mx.get("mask") or {}
                 mixer = PooledWindowAttention(
-                    W, int(mx["heads"]), int(mx["kv_heads"]), int(mx["dim"]),
-                    int(mx["vdim"]), float(mx["scale"]),
-                    float(mx.get("softcap", 0.0)), int(mask["size"]),
+                    W, int(mx["heads"]), int(mx.get("kv_heads", mx["heads"])), int(mx["dim"]),
+                    int(mx.get("vdim", mx["dim"])), float(mx["scale"]),
+                    float(mx.get("softcap") or 0.0), int(mask["size"]),
                     int(mask.get("pool", 0)), eps, idx, owns,
                 )
             else:

@@ -1,5 +1,7 @@
 """Sequence-mixer ops: layer norm over an fp32 residual stream, sliding-window
-attention over a compressed latent cache, gated linear attention.
+attention over a compressed latent cache, gated linear attention; sandwich
+RMS norm with depth-weighted averaging, row-cache attention (differential /
+pooled sliding window) and xIELU.
 
 GPU tensors go to the hand-written gfx950 kernels of the in-tree extension
 ``parallax_amd.ops._mix`` (bf16 or float32 activations; scores, norms, decays

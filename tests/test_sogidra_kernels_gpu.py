@@ -25,7 +25,7 @@ def _tol(dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
-@pytest.mark.parametrize("W", [40, 256, 1000, 4500])
+@pytest.mark.parametrize("W", [40, 46, 256, 1000, 4500])
 def test_sandwich_rmsnorm(dtype, W):
     T, n_max = 5, 4
     x = _rand(T, W, seed=1) + 0.3
